@@ -37,6 +37,12 @@ def first_visible(spec, position: int) -> int:
     return 0 if window is None else max(0, position + 1 - window)
 
 
+def kept_pages(spec, page_size: int) -> int:
+    """Logical pages at a sequence's start that are never given back while the request lives (a window that keeps
+    the first positions readable)."""
+    return -(-int(getattr(spec, "keep_first", 0) or 0) // page_size)
+
+
 def reach(spec) -> Optional[int]:
     """The most positions back (the query's own included) that any query reads, or ``None`` if there is no bound."""
     spans = [s for s in (getattr(spec, "window", None), getattr(spec, "chunk", None)) if s is not None]
@@ -198,7 +204,7 @@ class CacheManager:
         if window is None:
             return full
         # live keys span at most window - 1 + portion positions, which touch one page more
-        return min(full, -(-(window - 1 + portion) // self.page_size) + 1)
+        return min(full, -(-(window - 1 + portion) // self.page_size) + 1 + kept_pages(self.groups[group].spec, self.page_size))
 
     @property
     def free_slots(self) -> int:
@@ -281,7 +287,7 @@ class CacheManager:
             dead_below = min(first_needed // self.page_size, len(state.tables[g]))
             before = self._owed(state, g)
             dead = []
-            for logical in range(state.first_page[g], dead_below):
+            for logical in range(max(state.first_page[g], kept_pages(grp.spec, self.page_size)), dead_below):
                 if state.tables[g][logical] >= 0:
                     dead.append(state.tables[g][logical])
                     state.tables[g][logical] = -1

@@ -1,5 +1,5 @@
 // Generic paged attention: one wavefront per (token, query head), any head size up
-// to 512, any page size, fp32 or bf16 storage, all arithmetic in fp32.
+// to 1024, any page size, fp32 or bf16 storage, all arithmetic in fp32.
 //
 // Every token t of the packed batch belongs to request row token_row[t] and sees
 // the cached keys at positions [kv_lo[t], kv_hi[t]) of that row (kv_lo optional,
@@ -20,9 +20,17 @@
 //    element by element by the sigmoid of it;
 //  * a sink: one more term exp(sink_score) in the softmax's denominator that carries no value
 //    (has_sink != 0). The running maximum and sum then start from that term instead of from nothing.
+//    `sinks` (fp32 [H]) gives every head a score of its own for that term;
+//  * kept first keys: a query also sees the keys [0, min(keep_first, kv_lo)) of its row, before its window;
+//  * several maps per head (maps > 1): query heads and key heads come in groups of `maps` neighbours, map m of a
+//    query head reads map m of its key head, and all maps of a key head share one value head: H and Hkv count maps,
+//    the value cache has Hkv / maps heads;
+//  * values inside the keys (values_in_keys != 0): the value of a key is the first hdv channels of its key row
+//    (a cache of latents that are both); v_cache is then not read;
+//  * out_f32 != 0: the output is written as fp32 whatever the type of queries and cache.
 #include "ka_common.h"
 
-constexpr int ATT_MAX_HD = 512;
+constexpr int ATT_MAX_HD = 1024;
 
 // Four neighbouring elements with one load (the address must be a multiple of 4 elements).
 template <typename T>
@@ -43,12 +51,16 @@ attention_generic_kernel(const T* __restrict__ q, long q_row_stride, const T* __
                          int hd, int hdv, int page_size, const int* __restrict__ positions,
                          const float* __restrict__ slopes, int has_sink, float sink_score,
                          const float* __restrict__ bias_table, int bias_len, const T* __restrict__ gate,
-                         long gate_row_stride) {
+                         long gate_row_stride, const float* __restrict__ sinks, int keep_first, int maps,
+                         int values_in_keys, int out_f32) {
     __shared__ float qs[ATT_MAX_HD];
     __shared__ float ps[KA_WAVE];
     __shared__ long offs[KA_WAVE];   // value cache offset of channel 0 of each key of the chunk
     int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
-    int kvh = h / (H / Hkv);
+    // (maps == 1: query head h reads kv head h / (H / Hkv), keys and values alike)
+    const int vh = h / maps / (H / Hkv);
+    const int kvh = vh * maps + h % maps;
+    const int Hv = Hkv / maps;
     int row = token_row[t];
     int lo = kv_lo ? kv_lo[t] : 0, hi = kv_hi[t];
     const T* qp = q + (size_t)t * q_row_stride + (size_t)h * hd;
@@ -60,11 +72,15 @@ attention_generic_kernel(const T* __restrict__ q, long q_row_stride, const T* __
     const int* bt = block_table + (size_t)row * max_pages;
     const bool k_vectors = hd % 4 == 0 && reinterpret_cast<uintptr_t>(k_cache) % (4 * sizeof(T)) == 0;
     const bool v_vectors = page_size % 4 == 0 && reinterpret_cast<uintptr_t>(v_cache) % (4 * sizeof(T)) == 0;
+    if (sinks) sink_score = sinks[h];
     float m = has_sink ? sink_score : -INFINITY, l = has_sink ? 1.f : 0.f;
     float o[ATT_MAX_HD / KA_WAVE];
 #pragma unroll
     for (int i = 0; i < ATT_MAX_HD / KA_WAVE; ++i) o[i] = 0.f;
-    for (int base = lo; base < hi; base += KA_WAVE) {
+    const int kept = min(keep_first, lo);            // keys [0, kept) before the window, then [lo, hi)
+    for (int part = kept > 0 ? 0 : 1; part < 2; ++part)
+    for (int base = part ? lo : 0, hi_here = part ? hi : kept; base < hi_here; base += KA_WAVE) {
+        const int hi = hi_here;
         int key = base + lane;
         bool valid = key < hi;
         float s = -INFINITY;
@@ -72,7 +88,7 @@ attention_generic_kernel(const T* __restrict__ q, long q_row_stride, const T* __
         if (valid) {
             int page = bt[key / page_size];
             const T* kp = k_cache + (((long)page * Hkv + kvh) * page_size + key % page_size) * hd;
-            off = ((long)page * Hkv + kvh) * hdv * page_size + key % page_size;
+            off = values_in_keys ? (long)(kp - k_cache) : ((long)page * Hv + vh) * hdv * page_size + key % page_size;
             float acc = 0.f;
             if (k_vectors) {
                 // four channels with one load, added in the same order as one by one
@@ -103,12 +119,12 @@ attention_generic_kernel(const T* __restrict__ q, long q_row_stride, const T* __
             int d = lane + i * KA_WAVE;
             if (d < hdv) {
                 float acc = o[i] * corr;
-                const T* vd = v_cache + (long)d * page_size;
+                const T* vd = values_in_keys ? k_cache + d : v_cache + (long)d * page_size;
                 int j = 0;
                 // A chunk that starts on a multiple of four keys: every four keys from there lie in
                 // one page, their values side by side in the cache: one load, added in the same
                 // order as one by one.
-                if (v_vectors && (base & 3) == 0) {
+                if (v_vectors && !values_in_keys && (base & 3) == 0) {
                     for (; j + 3 < count; j += 4) {
                         float v4[4];
                         att_load4(vd + offs[j], v4);
@@ -122,7 +138,7 @@ attention_generic_kernel(const T* __restrict__ q, long q_row_stride, const T* __
         }
     }
     float inv = l > 0.f ? 1.0f / l : 0.f;
-    T* op = out + (size_t)t * out_row_stride + (size_t)h * hdv;
+    const size_t out_at = (size_t)t * out_row_stride + (size_t)h * hdv;
 #pragma unroll
     for (int i = 0; i < ATT_MAX_HD / KA_WAVE; ++i) {
         int d = lane + i * KA_WAVE;
@@ -130,7 +146,8 @@ attention_generic_kernel(const T* __restrict__ q, long q_row_stride, const T* __
             float y = o[i] * inv;
             // (an output gate: the head's channels times the sigmoid of the gate's pre-activations of the same token)
             if (gate) y *= 1.0f / (1.0f + expf(-ka_to_float(gate[(size_t)t * gate_row_stride + (size_t)h * hdv + d])));
-            op[d] = ka_from_float<T>(y);
+            if (out_f32) reinterpret_cast<float*>(out)[out_at + d] = y;
+            else out[out_at + d] = ka_from_float<T>(y);
         }
     }
 }
@@ -141,7 +158,11 @@ KA_API int ka_attention_generic(const void* q, int dtype, long q_row_stride, con
                                 long out_row_stride, float scale, int n, int H, int Hkv, int hd,
                                 int page_size, int hdv, const int* positions, const float* slopes,
                                 int has_sink, float sink_score, const float* bias_table, int bias_len,
-                                const void* gate, long gate_row_stride, hipStream_t stream) {
+                                const void* gate, long gate_row_stride, const float* sinks, int keep_first, int maps,
+                                int values_in_keys, int out_f32, hipStream_t stream) {
+    KA_CHECK(maps >= 1 && H % maps == 0 && Hkv % maps == 0 && keep_first >= 0, "ka_attention_generic: %d maps do not divide the heads %d and %d", maps, H, Hkv);
+    KA_CHECK(!values_in_keys || hdv <= hd, "ka_attention_generic: values inside keys of %d channels cannot have %d", hd, hdv);
+    KA_CHECK(sinks == nullptr || has_sink, "ka_attention_generic: sink scores without a sink");
     KA_CHECK(bias_table == nullptr || (positions != nullptr && bias_len > 0), "ka_attention_generic: a distance table needs the queries' positions");
     KA_CHECK(n >= 0 && H > 0 && Hkv > 0 && hd > 0 && hdv > 0, "ka_attention_generic: bad sizes");
     KA_CHECK(hdv <= ATT_MAX_HD, "ka_attention_generic: value size %d above %d", hdv, ATT_MAX_HD);
@@ -156,12 +177,12 @@ KA_API int ka_attention_generic(const void* q, int dtype, long q_row_stride, con
         hipLaunchKernelGGL(attention_generic_kernel<float>, grid, block, 0, stream, (const float*)q, q_row_stride,
                            (const float*)k_cache, (const float*)v_cache, block_table, max_pages, token_row, kv_lo,
                            kv_hi, (float*)out, out_row_stride, scale, H, Hkv, hd, hdv, page_size, positions, slopes, has_sink,
-                           sink_score, bias_table, bias_len, (const float*)gate, gate_row_stride);
+                           sink_score, bias_table, bias_len, (const float*)gate, gate_row_stride, sinks, keep_first, maps, values_in_keys, out_f32);
     else if (dtype == KA_BF16)
         hipLaunchKernelGGL(attention_generic_kernel<bf16_t>, grid, block, 0, stream, (const bf16_t*)q, q_row_stride,
                            (const bf16_t*)k_cache, (const bf16_t*)v_cache, block_table, max_pages, token_row, kv_lo,
                            kv_hi, (bf16_t*)out, out_row_stride, scale, H, Hkv, hd, hdv, page_size, positions, slopes, has_sink,
-                           sink_score, bias_table, bias_len, (const bf16_t*)gate, gate_row_stride);
+                           sink_score, bias_table, bias_len, (const bf16_t*)gate, gate_row_stride, sinks, keep_first, maps, values_in_keys, out_f32);
     else
         KA_CHECK(false, "ka_attention_generic: unsupported dtype %d", dtype);
     KA_LAUNCH_CHECK();

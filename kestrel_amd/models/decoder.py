@@ -88,6 +88,10 @@ class DecoderModel:
         for entry in self.plan.schedule:
             mixer = self.blocks[entry.layer].mixer
             needs.append((mixer.cache_spec(), mixer.state_spec(), entry.reads_cache_of))
+        # behind the schedule's entries: what parts outside the layers keep per request (no keys and values)
+        position_state = getattr(self.position, "state_spec", None)
+        if callable(position_state) and position_state() is not None:
+            needs.append((None, position_state(), None))
         return needs
 
     def position_axes(self) -> int:
@@ -130,7 +134,11 @@ class DecoderModel:
         if batch.given_embeds is not None:
             core.scatter_rows(batch.given_embeds, batch.given_rows, x)
         if self.position is not None:
-            self.position.add_to_embeddings(x, batch)
+            position_state = getattr(self.position, "state_spec", None)
+            if callable(position_state) and position_state() is not None:
+                self.position.add_to_embeddings(x, batch, state=caches[len(plan.schedule)].state)
+            else:
+                self.position.add_to_embeddings(x, batch)
         for junction in self.junctions.values():
             junction.begin(x, batch)
         handed = None      # the next block's first norm of x, where a block's last launch has computed it
@@ -141,7 +149,7 @@ class DecoderModel:
             before = getattr(entry, "before", None)
             if before is not None:
                 settle(x, batch)
-                self.junctions[before].forward(x, batch)
+                self.junctions[before].forward(x, batch, passage=int(getattr(entry, "passage", 0)))
                 handed = None
             handed = self.blocks[entry.layer].forward(x, batch, caches[index], normed=handed, then=then)
         settle(x, batch)       # (what the last block has left to be added into the stream)

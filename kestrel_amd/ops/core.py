@@ -31,12 +31,25 @@ _SIGNATURES = {
                           _c_long, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void_p],
     "ka_attention_generic": [_c_void_p, _c_int, _c_long, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_void_p,
                              _c_void_p, _c_void_p, _c_void_p, _c_long, _c_float, _c_int, _c_int, _c_int, _c_int,
-                             _c_int, _c_int, _c_void_p, _c_void_p, _c_int, _c_float, _c_void_p, _c_int, _c_void_p, _c_long, _c_void_p],
+                             _c_int, _c_int, _c_void_p, _c_void_p, _c_int, _c_float, _c_void_p, _c_int, _c_void_p, _c_long,
+                             _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_void_p],
     "ka_rmsnorm": [_c_void_p, _c_void_p, _c_void_p, _c_float, _c_void_p, _c_int, _c_int, _c_int, _c_void_p],
     "ka_qkv_prepare": [_c_void_p, _c_int, _c_long, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int,
                        _c_int, _c_int, _c_int, _c_void_p, _c_void_p, _c_float, _c_void_p, _c_int, _c_int, _c_float, _c_int,
                        _c_int, _c_void_p, _c_long, _c_void_p, _c_void_p],
     "ka_gated_pairs": [_c_void_p, _c_long, _c_void_p, _c_long, _c_int, _c_int, _c_int, _c_int, _c_void_p],
+    "ka_pair_embed": [_c_void_p, _c_int, _c_void_p, _c_void_p, _c_int, _c_int, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p,
+                      _c_int, _c_long, _c_long, _c_void_p, _c_int, _c_int, _c_int, _c_void_p],
+    "ka_conv_prepare": [_c_void_p, _c_int, _c_long, _c_void_p, _c_void_p, _c_int, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p,
+                        _c_void_p, _c_long, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int,
+                        _c_void_p, _c_int, _c_int, _c_void_p],
+    "ka_maps_combine": [_c_void_p, _c_void_p, _c_int, _c_long, _c_int, _c_int, _c_int, _c_float, _c_float, _c_float, _c_void_p],
+    "ka_latent_prepare": [_c_void_p, _c_int, _c_long, _c_int, _c_int, _c_void_p, _c_void_p, _c_int, _c_int, _c_void_p, _c_int,
+                          _c_void_p, _c_int, _c_int, _c_void_p, _c_void_p, _c_void_p, _c_float, _c_int, _c_void_p],
+    "ka_rotate_tail": [_c_void_p, _c_int, _c_long, _c_void_p, _c_long, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void_p, _c_int,
+                       _c_int, _c_void_p, _c_void_p],
+    "ka_clamped_pairs": [_c_void_p, _c_long, _c_void_p, _c_long, _c_int, _c_int, _c_int, _c_float, _c_float, _c_float, _c_void_p],
+    "ka_add_vector": [_c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_void_p],
     "ka_gate_mul": [_c_void_p, _c_long, _c_void_p, _c_long, _c_int, _c_int, _c_int, _c_void_p],
     "ka_branches_sum": [_c_void_p, _c_void_p, _c_void_p, _c_float, _c_void_p, _c_void_p, _c_float, _c_float, _c_int, _c_int,
                         _c_void_p],
@@ -405,6 +418,159 @@ def gated_pairs(x: torch.Tensor, out: torch.Tensor, act: int) -> None:
                                 code_of(x.dtype), n, n_out, int(act), stream_ptr()))
 
 
+def clamped_pairs(x: torch.Tensor, out: torch.Tensor, limit: float, slope: float, shift: float) -> None:
+    """``out[:, j] = g sigmoid(slope g) (u + shift)`` with ``g = min(x[:, 2 j], limit)`` and ``u = clamp(x[:, 2 j + 1], -limit, limit)``:
+    the product of the pairs that a plain linear over paired weight rows (``ops.linear.pair_rows``) leaves side by side."""
+    _dev(x, out)
+    n, n_out = out.shape
+    _need(x.dim() == 2 and tuple(x.shape) == (n, 2 * n_out) and x.dtype == out.dtype and x.stride(1) == 1 and out.stride(1) == 1,
+          "clamped_pairs: x must be [n, 2 m] and out [n, m] of one type")
+    _check(lib().ka_clamped_pairs(x.data_ptr(), x.stride(0) if n > 1 else 2 * n_out, out.data_ptr(), out.stride(0) if n > 1 else n_out,
+                                  code_of(x.dtype), n, n_out, float(limit), float(slope), float(shift), stream_ptr()))
+
+
+def add_vector(x: torch.Tensor, vector: torch.Tensor) -> None:
+    """``x[t] += vector`` for every row of fp32 ``x`` ``[n, dim]``."""
+    _dev(x, vector)
+    n, dim = x.shape
+    _need(x.dtype == torch.float32 and x.is_contiguous() and vector.numel() == dim and vector.is_contiguous(),
+          "add_vector: x must be contiguous fp32 [n, dim] and the vector [dim]")
+    _check(lib().ka_add_vector(x.data_ptr(), vector.data_ptr(), code_of(vector.dtype), n, dim, stream_ptr()))
+
+
+def pair_embed(table: torch.Tensor, ids: torch.Tensor, positions: torch.Tensor, token_row: torch.Tensor, cu_q: torch.Tensor,
+               row_slot: torch.Tensor, last_token: torch.Tensor, buckets: int, mul_prev: int, mul_cur: int, x: torch.Tensor,
+               vocab: int, pending: Optional[torch.Tensor] = None) -> None:
+    """``x[t] += table[(prev mul_prev + cur mul_cur) mod buckets]`` for every token with the token before it in its
+    sequence, ``table[buckets]`` for a sequence's first token. The token before a row's first token of this step is
+    ``last_token[slot]`` (int32 ``[slots + 1]``), which is then set to the row's last token. Ids as ``embed`` takes them."""
+    _dev(table, ids, positions, token_row, cu_q, row_slot, last_token, x, pending)
+    n, dim = x.shape
+    n_rows = row_slot.numel()
+    _need(table.dim() == 2 and table.shape[0] == buckets + 1 and table.shape[1] == dim and table.is_contiguous(),
+          "pair_embed: table must be [buckets + 1, dim]")
+    _need(x.dtype == torch.float32 and x.is_contiguous(), "pair_embed: x must be contiguous fp32")
+    for t in (ids, positions, token_row):
+        _need(t.dtype == torch.int32 and t.numel() == n and t.is_contiguous(), "pair_embed: per-token int32 [n] expected")
+    _need(cu_q.dtype == torch.int32 and cu_q.numel() == n_rows + 1 and row_slot.dtype == torch.int32 and cu_q.is_contiguous()
+          and row_slot.is_contiguous(), "pair_embed: cu_q int32 [rows + 1] and row_slot int32 [rows]")
+    _need(last_token.dtype == torch.int32 and last_token.is_contiguous(), "pair_embed: last_token must be int32")
+    _need(pending is None or (pending.dtype == torch.int32 and pending.is_contiguous()), "pair_embed: pending must be int32")
+    _check(lib().ka_pair_embed(table.data_ptr(), code_of(table.dtype), ids.data_ptr(), _ptr(pending),
+                               0 if pending is None else pending.numel(), int(vocab), positions.data_ptr(), token_row.data_ptr(),
+                               cu_q.data_ptr(), row_slot.data_ptr(), last_token.data_ptr(), int(buckets), int(mul_prev), int(mul_cur),
+                               x.data_ptr(), n, n_rows, dim, stream_ptr()))
+
+
+def conv_prepare(u: torch.Tensor, taps: Optional[torch.Tensor], state: Optional[torch.Tensor], cu_q: torch.Tensor,
+                 row_slot: torch.Tensor, token_row: torch.Tensor, positions: torch.Tensor, slots: Optional[torch.Tensor],
+                 q_out: torch.Tensor, k_cache: Optional[torch.Tensor], v_cache: Optional[torch.Tensor], q_heads: int, k_heads: int,
+                 head_dim: int, v_heads: int, value_dim: int, page_size: int, freqs: Optional[torch.Tensor] = None,
+                 pairing: str = "halves") -> None:
+    """A short causal convolution over time on every channel of the projected rows ``u`` ``[n, q | k | v]``
+    (``taps`` fp32 ``[channels, K]``: ``y_t = sum_j taps[:, j] u_(t - K + 1 + j)``; ``None``: none), then the rotation of the
+    first ``2 len(freqs)`` channels of every query and key head by ``place * freqs``, then queries into ``q_out`` ``[n, q]``,
+    keys into the paged ``k_cache`` ``[pages, k_heads, page, hd]`` and values into ``v_cache`` ``[pages, v_heads, hdv, page]`` at
+    ``slots``. Inputs from before this step come from ``state`` fp32 ``[slots + 1, K - 1, channels]`` (by ``row_slot``), which is
+    then moved on to the last ``K - 1`` rows of ``u`` of every row."""
+    _need(pairing in ROTARY_PAIRINGS, f"conv_prepare: pairing {pairing!r} is not one of {sorted(ROTARY_PAIRINGS)}")
+    _dev(u, taps, state, cu_q, row_slot, token_row, positions, slots, q_out, k_cache, v_cache, freqs)
+    n = u.shape[0]
+    channels = (q_heads + k_heads) * head_dim + v_heads * value_dim
+    _need(u.dim() == 2 and u.stride(1) == 1 and u.shape[1] == channels, "conv_prepare: u must be [n, q + k + v]")
+    _need(q_out.dim() == 2 and q_out.stride(1) == 1 and tuple(q_out.shape) == (n, q_heads * head_dim) and q_out.dtype == u.dtype,
+          "conv_prepare: q_out must be [n, q] of the type of u")
+    K = 0
+    if taps is not None:
+        _need(taps.dtype == torch.float32 and taps.dim() == 2 and taps.shape[0] == channels and taps.is_contiguous(),
+              "conv_prepare: taps must be fp32 [channels, K]")
+        K = int(taps.shape[1])
+        _need(K >= 1, "conv_prepare: at least one tap")
+    n_rows = row_slot.numel()
+    if K > 1:
+        _need(state is not None and state.dtype == torch.float32 and state.is_contiguous() and tuple(state.shape[1:]) == (K - 1, channels),
+              "conv_prepare: state must be fp32 [slots + 1, K - 1, channels]")
+    for t in (token_row, positions) + ((slots,) if slots is not None else ()):
+        _need(t.dtype == torch.int32 and t.numel() == n and t.is_contiguous(), "conv_prepare: per-token int32 [n] expected")
+    _need(cu_q.dtype == torch.int32 and cu_q.numel() == n_rows + 1 and cu_q.is_contiguous() and row_slot.dtype == torch.int32
+          and row_slot.is_contiguous(), "conv_prepare: cu_q int32 [rows + 1] and row_slot int32 [rows]")
+    if slots is not None:
+        _need(k_cache is not None and v_cache is not None and k_cache.dtype == u.dtype and v_cache.dtype == u.dtype
+              and k_cache.is_contiguous() and v_cache.is_contiguous()
+              and tuple(k_cache.shape[1:]) == (k_heads, page_size, head_dim)
+              and tuple(v_cache.shape[1:]) == (v_heads, value_dim, page_size), "conv_prepare: caches [pages, Hk, page, hd] and [pages, Hv, hdv, page]")
+    rot = 0
+    if freqs is not None:
+        _need(freqs.dtype == torch.float32 and freqs.dim() == 1 and freqs.is_contiguous(), "conv_prepare: freqs fp32 [R / 2]")
+        rot = 2 * freqs.numel()
+    _check(lib().ka_conv_prepare(u.data_ptr(), code_of(u.dtype), u.stride(0) if n > 1 else channels, _ptr(taps), _ptr(state) if K > 1 else None, K,
+                                 cu_q.data_ptr(), row_slot.data_ptr(), token_row.data_ptr(), positions.data_ptr(), _ptr(slots),
+                                 q_out.data_ptr(), q_out.stride(0) if n > 1 else q_heads * head_dim, _ptr(k_cache), _ptr(v_cache), n, n_rows,
+                                 q_heads, k_heads, head_dim, v_heads, value_dim, page_size, _ptr(freqs), rot, ROTARY_PAIRINGS[pairing],
+                                 stream_ptr()))
+
+
+def maps_combine(maps: torch.Tensor, out: torch.Tensor, n_heads: int, value_dim: int, weight: float, eps: float, out_scale: float) -> None:
+    """``maps`` fp32 ``[n, H 2 hdv]``, two attentions per head over the same values: ``o = a1 - weight a2``, then
+    ``o / sqrt(mean(o^2) + eps) * out_scale`` over a head's values, into ``out`` ``[n, H hdv]``."""
+    _dev(maps, out)
+    n = out.shape[0]
+    _need(maps.dtype == torch.float32 and maps.is_contiguous() and tuple(maps.shape) == (n, 2 * n_heads * value_dim),
+          "maps_combine: maps must be contiguous fp32 [n, H 2 hdv]")
+    _need(out.dim() == 2 and out.stride(1) == 1 and out.shape[1] == n_heads * value_dim, "maps_combine: out must be [n, H hdv]")
+    _check(lib().ka_maps_combine(maps.data_ptr(), out.data_ptr(), code_of(out.dtype), out.stride(0) if n > 1 else n_heads * value_dim, n,
+                                 n_heads, value_dim, float(weight), float(eps), float(out_scale), stream_ptr()))
+
+
+def latent_prepare(down: torch.Tensor, q_at: int, q_rank: int, q_gain: Optional[torch.Tensor], cq: Optional[torch.Tensor], kv_at: int,
+                   rank: int, kv_gain: Optional[torch.Tensor], rot_dim: int, freqs: Optional[torch.Tensor], pairing: str,
+                   positions: torch.Tensor, slots: Optional[torch.Tensor], cache: Optional[torch.Tensor], eps: float) -> None:
+    """Latents of a step made ready: the query latent ``down[:, q_at : q_at + q_rank]`` normalised (root mean square, gains)
+    into ``cq`` ``[n, q_rank]``; the key/value latent ``down[:, kv_at : kv_at + rank]`` normalised the same way and the ``rot_dim``
+    channels behind it rotated by ``place * freqs`` side by side into the paged ``cache`` ``[pages, 1, page, rank + rot_dim]`` at
+    ``slots``."""
+    _need(pairing in ROTARY_PAIRINGS, f"latent_prepare: pairing {pairing!r} is not one of {sorted(ROTARY_PAIRINGS)}")
+    _dev(down, q_gain, cq, kv_gain, freqs, positions, slots, cache)
+    n = down.shape[0]
+    _need(down.dim() == 2 and down.stride(1) == 1, "latent_prepare: rows must be contiguous")
+    if q_rank:
+        _need(cq is not None and cq.dtype == down.dtype and cq.is_contiguous() and tuple(cq.shape) == (n, q_rank), "latent_prepare: cq must be [n, q_rank]")
+    for gain, size in ((q_gain, q_rank), (kv_gain, rank)):
+        _need(gain is None or (gain.dtype == torch.float32 and gain.numel() == size and gain.is_contiguous()), "latent_prepare: gains fp32")
+    for t in (positions,) + ((slots,) if slots is not None else ()):
+        _need(t.dtype == torch.int32 and t.numel() == n and t.is_contiguous(), "latent_prepare: per-token int32 [n] expected")
+    if slots is not None:
+        _need(cache is not None and cache.dtype == down.dtype and cache.is_contiguous() and cache.dim() == 4 and cache.shape[1] == 1
+              and cache.shape[3] == rank + rot_dim, "latent_prepare: cache must be [pages, 1, page, rank + rot_dim]")
+    rot = 0
+    if freqs is not None:
+        _need(freqs.dtype == torch.float32 and freqs.dim() == 1 and freqs.is_contiguous(), "latent_prepare: freqs fp32 [R / 2]")
+        rot = 2 * freqs.numel()
+    _check(lib().ka_latent_prepare(down.data_ptr(), code_of(down.dtype), down.stride(0) if n > 1 else down.shape[1], int(q_at), int(q_rank),
+                                   _ptr(q_gain), _ptr(cq), int(kv_at), int(rank), _ptr(kv_gain), int(rot_dim), _ptr(freqs), rot,
+                                   ROTARY_PAIRINGS[pairing], positions.data_ptr(), _ptr(slots), _ptr(cache), float(eps), n, stream_ptr()))
+
+
+def rotate_tail(src: torch.Tensor, dst: torch.Tensor, n_heads: int, plain_dim: int, rot_dim: int, rank: int,
+                freqs: Optional[torch.Tensor], pairing: str, positions: torch.Tensor) -> None:
+    """``src`` ``[n, H (plain_dim + rot_dim)]`` -> ``dst`` ``[n, H (rank + rot_dim)]``: the last ``rot_dim`` channels of every head,
+    rotated by ``place * freqs``, written behind the first ``rank`` channels of the head in ``dst`` (which are left alone)."""
+    _need(pairing in ROTARY_PAIRINGS, f"rotate_tail: pairing {pairing!r} is not one of {sorted(ROTARY_PAIRINGS)}")
+    _dev(src, dst, freqs, positions)
+    n = src.shape[0]
+    _need(src.dim() == 2 and src.stride(1) == 1 and src.shape[1] == n_heads * (plain_dim + rot_dim) and dst.dim() == 2
+          and dst.stride(1) == 1 and tuple(dst.shape) == (n, n_heads * (rank + rot_dim)) and dst.dtype == src.dtype,
+          "rotate_tail: src [n, H (d + dr)] and dst [n, H (rank + dr)] of one type")
+    _need(positions.dtype == torch.int32 and positions.numel() == n and positions.is_contiguous(), "rotate_tail: positions int32 [n]")
+    rot = 0
+    if freqs is not None:
+        _need(freqs.dtype == torch.float32 and freqs.dim() == 1 and freqs.is_contiguous(), "rotate_tail: freqs fp32 [R / 2]")
+        rot = 2 * freqs.numel()
+    _check(lib().ka_rotate_tail(src.data_ptr(), code_of(src.dtype), src.stride(0) if n > 1 else src.shape[1], dst.data_ptr(),
+                                dst.stride(0) if n > 1 else dst.shape[1], n, n_heads, plain_dim, rot_dim, rank, _ptr(freqs), rot,
+                                ROTARY_PAIRINGS[pairing], positions.data_ptr(), stream_ptr()))
+
+
 def gate_mul(x: torch.Tensor, gate: torch.Tensor) -> None:
     """``x *= sigmoid(gate)`` element by element; both ``[n, dim]`` of one type, rows may lie in wider buffers."""
     _dev(x, gate)
@@ -528,8 +694,16 @@ def attention_generic(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Ten
                       out: torch.Tensor, scale: float, n_heads: int, n_kv_heads: int, head_dim: int,
                       value_dim: Optional[int] = None, positions: Optional[torch.Tensor] = None,
                       slopes: Optional[torch.Tensor] = None, sink: Optional[float] = None,
-                      bias_table: Optional[torch.Tensor] = None, gate: Optional[torch.Tensor] = None) -> None:
+                      bias_table: Optional[torch.Tensor] = None, gate: Optional[torch.Tensor] = None,
+                      sinks: Optional[torch.Tensor] = None, keep_first: int = 0, maps: int = 1,
+                      values_in_keys: bool = False) -> None:
     """Paged attention of ``n`` packed tokens; ``q`` may be a strided view into a qkv buffer.
+
+    ``sinks`` (fp32 ``[H]``): a score per head for the valueless term instead of the one number ``sink``. ``keep_first``: a
+    query also sees the first ``keep_first`` keys of its row where its window (``kv_lo``) has passed them. ``maps`` > 1:
+    query and key heads come in groups of ``maps`` neighbours that share one value head (``n_heads`` and ``n_kv_heads``
+    count maps; the value cache has ``n_kv_heads / maps`` heads). ``values_in_keys``: a key's value is the first
+    ``value_dim`` channels of its key row (``v_cache`` is ``None``). ``out`` may be fp32 where ``q`` is not.
 
     ``value_dim``: size of a value head where it differs from ``head_dim`` (``out`` is ``[n, H value_dim]``).
     ``slopes`` (fp32 ``[H]``) with ``positions`` (int32 ``[n]``): the score of a query at place ``i`` against the key
@@ -541,10 +715,24 @@ def attention_generic(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Ten
     n = q.shape[0]
     value_dim = head_dim if value_dim is None else int(value_dim)
     _need(q.dim() == 2 and q.stride(1) == 1 and q.shape[1] >= n_heads * head_dim, "attention: q must be [n, >= H hd]")
-    _need(out.dim() == 2 and out.stride(1) == 1 and tuple(out.shape) == (n, n_heads * value_dim) and out.dtype == q.dtype,
-          "attention: out must be [n, H hdv] of the q type")
+    _need(out.dim() == 2 and out.stride(1) == 1 and tuple(out.shape) == (n, n_heads * value_dim)
+          and out.dtype in (q.dtype, torch.float32), "attention: out must be [n, H hdv] of the q type or fp32")
     page_size = k_cache.shape[2]
-    _check_caches("attention", k_cache, v_cache, q.dtype, n_kv_heads, page_size, head_dim, value_dim)
+    maps = int(maps)
+    _need(maps >= 1 and n_heads % maps == 0 and n_kv_heads % maps == 0, "attention: the maps must divide the heads")
+    if values_in_keys:
+        _need(v_cache is None and value_dim <= head_dim and k_cache.dtype == q.dtype and k_cache.is_contiguous()
+              and tuple(k_cache.shape[1:]) == (n_kv_heads, page_size, head_dim), "attention: keys that hold their values: [pages, Hkv, page, hd]")
+    elif maps > 1:
+        _need(k_cache.dtype == q.dtype and k_cache.is_contiguous() and tuple(k_cache.shape[1:]) == (n_kv_heads, page_size, head_dim)
+              and v_cache.dtype == q.dtype and v_cache.is_contiguous()
+              and tuple(v_cache.shape) == (k_cache.shape[0], n_kv_heads // maps, value_dim, page_size),
+              "attention: with maps, keys [pages, Hkv, page, hd] and values [pages, Hkv / maps, hdv, page]")
+    else:
+        _check_caches("attention", k_cache, v_cache, q.dtype, n_kv_heads, page_size, head_dim, value_dim)
+    if sinks is not None:
+        _need(sinks.is_cuda and sinks.dtype == torch.float32 and sinks.numel() == n_heads and sinks.is_contiguous(),
+              "attention: sink scores must be fp32 [H]")
     if slopes is not None:
         _need(slopes.dtype == torch.float32 and slopes.numel() == n_heads and slopes.is_contiguous(),
               "attention: slopes must be fp32 [H]")
@@ -562,13 +750,15 @@ def attention_generic(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Ten
     for t in (token_row, kv_hi) + ((kv_lo,) if kv_lo is not None else ()):
         _need(t.dtype == torch.int32 and t.numel() == n and t.is_contiguous(), "attention: per-token int32 [n] expected")
     _check(lib().ka_attention_generic(q.data_ptr(), code_of(q.dtype), q.stride(0), k_cache.data_ptr(),
-                                      v_cache.data_ptr(), block_table.data_ptr(), block_table.shape[1],
+                                      _ptr(v_cache), block_table.data_ptr(), block_table.shape[1],
                                       token_row.data_ptr(), _ptr(kv_lo), kv_hi.data_ptr(), out.data_ptr(),
                                       out.stride(0), float(scale), n, n_heads, n_kv_heads, head_dim, page_size,
                                       value_dim, _ptr(positions) if (slopes is not None or bias_table is not None) else None,
-                                      _ptr(slopes), int(sink is not None), float(sink or 0.0), _ptr(bias_table),
+                                      _ptr(slopes), int(sink is not None or sinks is not None), float(sink or 0.0), _ptr(bias_table),
                                       int(bias_table.shape[1]) if bias_table is not None else 0, _ptr(gate),
-                                      (gate.stride(0) if n > 1 else n_heads * value_dim) if gate is not None else 0, stream_ptr()))
+                                      (gate.stride(0) if n > 1 else n_heads * value_dim) if gate is not None else 0,
+                                      _ptr(sinks), int(keep_first), maps, int(bool(values_in_keys)),
+                                      int(out.dtype == torch.float32 and q.dtype != torch.float32), stream_ptr()))
 
 
 def _pending_args(who: str, rows: int, pending, pending_at):

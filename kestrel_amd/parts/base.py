@@ -95,23 +95,30 @@ class PositionEncoding(Part):
     def rotation(self, device: torch.device) -> Optional[Rotation]:
         return None
 
-    def add_to_embeddings(self, x: torch.Tensor, batch) -> None:
+    def state_spec(self) -> Optional[StateSpec]:
+        """Model-level encodings: fixed-size state kept per request (something of the tokens before), or ``None``.
+        The cache manager keeps it like a mixer's; ``add_to_embeddings`` is then given it as ``state``."""
+        return None
+
+    def add_to_embeddings(self, x: torch.Tensor, batch, state: Optional[torch.Tensor] = None) -> None:
         """Model-level encodings: add the encoding of every token's position into the fp32 rows ``x``
         ``[tokens, dim]`` in place (``batch.positions``, ``batch.position_axes``). Under replayed graphs
-        (``batch.decode_only``) this must neither synchronise nor allocate."""
+        (``batch.decode_only``) this must neither synchronise nor allocate. ``state``: ``[slots + 1, *shape]``
+        of the encoding's ``state_spec``, indexed by ``batch.row_slot``."""
 
 
 class Junction(Part):
     """A transformation of the whole residual stream between two runs of layers (``ScheduleEntry.before``).
 
     ``begin`` is called once a step with the embedding output (after the model's position encoding), before the
-    first run; ``forward`` replaces fp32 ``x`` in place at every place of the schedule that names the junction.
-    Both must keep the promises of ``Part`` under replayed graphs."""
+    first run; ``forward`` replaces fp32 ``x`` in place at every place of the schedule that names the junction
+    (``passage``: the schedule entry's number for this passage). Both must keep the promises of ``Part`` under
+    replayed graphs."""
 
     def begin(self, x: torch.Tensor, batch) -> None:
         """See the embedding output ``x`` ``[tokens, dim]`` of this step."""
 
-    def forward(self, x: torch.Tensor, batch) -> None:
+    def forward(self, x: torch.Tensor, batch, passage: int = 0) -> None:
         raise NotImplementedError
 
 

@@ -102,12 +102,13 @@ _parallel.hands_over = True
 
 
 def _sequential(block: "Block", x, batch, cache) -> None:
-    """``x += mixer(norm(x)); x += ff(norm2(x))``."""
+    """``x += mixer(norm(x)); x += ff(norm2(x))``; without a feed-forward the first half only."""
     h = batch.workspace.get("block.h", tuple(x.shape), block.dtype)
     block.norm.forward(x, h)
     block.mixer.forward(h, batch, cache, x)
-    block.norm2.forward(x, h)
-    block.feed_forward.forward(h, batch, x)
+    if block.feed_forward is not None:
+        block.norm2.forward(x, h)
+        block.feed_forward.forward(h, batch, x)
 
 
 # Whether a block of weighted branches leaves the sum ``x += scale * delta`` to whoever reads the stream next (the
@@ -227,10 +228,10 @@ class Block:
         self.spec = spec
         self.norm = build_part("norm", spec.norm)
         self.norm2 = build_part("norm", spec.norm2) if spec.norm2 is not None else None
-        if spec.arrangement == "sequential" and self.norm2 is None:
-            raise ValueError("the sequential arrangement needs norm2")
+        if spec.arrangement == "sequential" and self.norm2 is None and spec.feed_forward is not None:
+            raise ValueError("the sequential arrangement needs norm2 for its feed-forward")
         self.mixer = build_part("mixer", spec.mixer)
-        if spec.feed_forward is None and spec.arrangement not in ("parallel_two_norms", "parallel"):
+        if spec.feed_forward is None and spec.arrangement not in ("parallel_two_norms", "parallel", "sequential"):
             raise ValueError(f"the {spec.arrangement} arrangement needs a feed-forward")
         if spec.arrangement == "parallel_two_norms" and spec.feed_forward is not None and self.norm2 is None:
             raise ValueError("the parallel_two_norms arrangement needs norm2 for its feed-forward")

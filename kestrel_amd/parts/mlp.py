@@ -8,7 +8,7 @@ import torch
 
 from ..ops.linear import ACT_GATED, activation_code, linear, linear_gated, pair_rows
 from .base import FeedForward, register_feed_forward
-from .specs import DenseFeedForwardSpec, GatedFeedForwardSpec, ParamSpec
+from .specs import ClampedGatedFeedForwardSpec, DenseFeedForwardSpec, GatedFeedForwardSpec, ParamSpec
 
 
 class DenseFeedForward(FeedForward):
@@ -108,5 +108,35 @@ class GatedFeedForward(FeedForward):
         linear(hidden, self.down_weight, self.down_bias, residual, accumulate=True)
 
 
+class ClampedGatedFeedForward(GatedFeedForward):
+    """``down(g sigmoid(slope g) (u + shift))`` with ``g = min(gate h, limit)`` and ``u = clamp(up h, -limit, limit)``.
+
+    The rows of ``gate`` and ``up`` are paired as in ``GatedFeedForward``; one plain linear computes both sums side by side
+    and a pass over them takes the clamps and the product (``ops.core.clamped_pairs``): the constants are numbers of the
+    layer, which the epilogues of the linear kernels (activations by code) do not carry."""
+
+    def __init__(self, spec: ClampedGatedFeedForwardSpec) -> None:
+        super().__init__(spec)
+        if not spec.limit > 0:
+            raise ValueError(f"the clamps of a gated feed-forward need a positive limit, got {spec.limit}")
+
+    def input_projection(self):
+        return None        # (no stage of this feed-forward is a linear with an activation by code)
+
+    def output_projection(self):
+        return None
+
+    def forward(self, h, batch, residual) -> None:
+        from ..ops import core
+        spec = self.spec
+        n = h.shape[0]
+        sums = batch.workspace.get("ff.pair_sums", (n, 2 * spec.hidden_dim), self.dtype)
+        hidden = batch.workspace.get("ff.hidden", (n, spec.hidden_dim), self.dtype)
+        linear(h, self.pairs, self.pair_bias, sums)
+        core.clamped_pairs(sums, hidden, spec.limit, spec.slope, spec.shift)
+        linear(hidden, self.down_weight, self.down_bias, residual, accumulate=True)
+
+
 register_feed_forward("dense", DenseFeedForward)
+register_feed_forward("clamped_gated_dense", ClampedGatedFeedForward)
 register_feed_forward("gated_dense", GatedFeedForward)

@@ -180,6 +180,11 @@ class CacheSpec:
     window: Optional[int] = None
     value_dim: Optional[int] = None     # size of a value head where it is not the keys' (``None``: ``head_dim``)
     chunk: Optional[int] = None
+    # the first ``keep_first`` positions of a sequence stay readable after a window has passed them: their pages are
+    # never given back while the request lives (``first_visible`` still names the window's start)
+    keep_first: int = 0
+    # value heads where they are fewer than key heads (several maps of keys over one head of values; ``None``: as many)
+    value_heads: Optional[int] = None
 
     def first_visible(self, position: int) -> int:
         """The lowest key position that a query at ``position`` reads."""
@@ -199,13 +204,33 @@ class CacheSpec:
         # values are kept transposed inside a page: eight consecutive keys of one channel are 16
         # bytes, which is what the MFMA attention kernels load at a time
         value_dim = self.head_dim if self.value_dim is None else self.value_dim
-        return {"k": (self.n_kv_heads, page_size, self.head_dim), "v": (self.n_kv_heads, value_dim, page_size)}
+        value_heads = self.n_kv_heads if self.value_heads is None else self.value_heads
+        return {"k": (self.n_kv_heads, page_size, self.head_dim), "v": (value_heads, value_dim, page_size)}
 
     @property
     def group_key(self) -> Tuple:
         value_dim = self.head_dim if self.value_dim is None else self.value_dim
         return ("kv", self.n_kv_heads, self.head_dim, self.window) + ((value_dim,) if value_dim != self.head_dim else ()) \
-            + ((("chunk", self.chunk),) if self.chunk is not None else ())
+            + ((("chunk", self.chunk),) if self.chunk is not None else ()) \
+            + ((("keep_first", self.keep_first),) if self.keep_first else ()) \
+            + ((("value_heads", self.value_heads),) if self.value_heads is not None else ())
+
+
+@dataclass(frozen=True)
+class LatentCacheSpec:
+    """What a latent attention mixer keeps per token: one row of ``latent_dim + shared_dim`` channels, the normalised
+    key/value latent and the rotated key part that all heads share, side by side (the row is key and value at once)."""
+
+    latent_dim: int
+    shared_dim: int
+    window: Optional[int] = None
+
+    def page_tensors(self, page_size: int) -> Dict[str, Tuple[int, ...]]:
+        return {"k": (1, page_size, self.latent_dim + self.shared_dim)}
+
+    @property
+    def group_key(self) -> Tuple:
+        return ("latent", self.latent_dim, self.shared_dim, self.window)
 
 
 @dataclass(frozen=True)
@@ -250,6 +275,98 @@ class AttentionSpec:
     value_blend: Optional[ValueBlend] = None
     # the concatenated heads multiplied by ``sigmoid(gate.weight @ input)`` before the output projection
     output_gate: bool = False
+
+
+@dataclass(frozen=True)
+class WindowWithKeptFirst:
+    """A query at place ``i`` reads the keys ``j <= i`` with ``i - j < size`` and, whatever their distance, the keys
+    ``j < keep_first``; kept keys stand at their true places."""
+
+    size: int
+    keep_first: int = 0
+
+
+@dataclass(frozen=True)
+class DifferentialAttentionSpec:
+    """Attention whose heads each hold two softmax maps over the same values, with queries ``[H, 2, head_dim]`` and keys
+    ``[G, 2, head_dim]`` laid out head by head as ``[map 1, map 2]``, combined as ``a1 - lambda a2`` with
+    ``lambda = exp(lq1 . lk1) - exp(lq2 . lk2) + lambda_init`` (one number for the layer), then divided by the root mean square
+    over a head's values (``eps``, no gain) and multiplied by ``1 - lambda_init``. ``conv_taps``: a causal convolution over
+    time on every channel of q, k and v right after their projections (``None``: none); ``mask`` ``None``: every ``j <= i``."""
+
+    kind: str
+    dim: int
+    n_heads: int
+    n_kv_heads: int
+    head_dim: int
+    value_dim: int
+    scale: float
+    lambda_init: float
+    eps: float
+    position: PositionSpec
+    conv_taps: Optional[int] = None
+    mask: Optional[WindowWithKeptFirst] = None
+
+
+@dataclass(frozen=True)
+class LatentAttentionSpec:
+    """Attention whose queries, keys and values come from low-rank latents: ``c_q = rms(W_dq h) g_q`` (``q_rank``),
+    ``q = W_uq c_q`` laid out per head as ``[head_dim plain, rot_dim rotated]``; ``W_dkv h`` gives the latent ``c`` (``kv_rank``,
+    normalised with gains) and ``rot_dim`` channels of one rotated key part shared by all heads; a head's plain keys are
+    ``W_uk c`` and its values ``W_uv c``. Every ``j <= i`` is seen. ``head_sinks``: one learned score per head that enters the
+    softmax's denominator without a value. ``output_gate``: the heads times ``sigmoid(W_g h)`` before the output
+    projection. ``position`` turns the ``rot_dim`` part."""
+
+    kind: str
+    dim: int
+    n_heads: int
+    head_dim: int
+    rot_dim: int
+    value_dim: int
+    q_rank: int
+    kv_rank: int
+    scale: float
+    eps: float
+    position: PositionSpec
+    head_sinks: bool = True
+    output_gate: bool = True
+
+
+@dataclass(frozen=True)
+class ClampedGatedFeedForwardSpec:
+    """``down(g sigmoid(slope g) (u + shift))`` with ``g = min(gate h, limit)`` and ``u = clamp(up h, -limit, limit)``."""
+
+    kind: str
+    dim: int
+    hidden_dim: int
+    limit: float
+    slope: float = 1.702
+    shift: float = 1.0
+    activation: str = "none"
+    bias: bool = False
+
+
+@dataclass(frozen=True)
+class PairEmbeddingSpec:
+    """An embedding of token pairs added to the embedded tokens: row ``(prev * mul_prev + cur * mul_cur) mod buckets`` of a
+    table of ``buckets + 1`` rows, and its last row for the first token of a sequence."""
+
+    kind: str
+    dim: int
+    buckets: int
+    mul_prev: int
+    mul_cur: int
+    vocab_size: int
+
+
+@dataclass(frozen=True)
+class PassVectorSpec:
+    """A junction that adds a learned vector to the stream, one vector per passage (``[passages, dim]``;
+    ``ScheduleEntry.passage`` says which)."""
+
+    kind: str
+    dim: int
+    passages: int
 
 
 @dataclass(frozen=True)
@@ -304,7 +421,7 @@ class LayerSpec:
     """One block: its parts, how they are arranged, and where their tensors are named.
 
     ``arrangement``: ``parallel`` = ``x + mixer(norm(x)) + ff(norm(x))`` (one norm; ``feed_forward`` may be ``None``);
-    ``sequential`` = ``x += mixer(norm(x)); x += ff(norm2(x))``;
+    ``sequential`` = ``x += mixer(norm(x)); x += ff(norm2(x))`` (``feed_forward`` and ``norm2`` may be ``None``: a mixer alone);
     ``parallel_two_norms`` = ``x + residual_scale * (mixer(norm(x)) + ff(norm2(x)))``, both norms of the same ``x``
     (``feed_forward`` and ``norm2`` may be ``None`` there: a layer of a mixer alone).
     ``names`` maps ``"<part>.<local tensor name>"`` (parts: ``norm``, ``norm2``, ``mixer``,
@@ -324,11 +441,13 @@ class LayerSpec:
 class ScheduleEntry:
     """One run of a layer. ``reads_cache_of``: index of an earlier schedule entry whose
     cache this run reads instead of keeping one of its own. ``before``: name of a junction of the
-    plan (``ModelPlan.junctions``) that the residual stream passes through right before this run."""
+    plan (``ModelPlan.junctions``) that the residual stream passes through right before this run; ``passage``: which
+    passage through that junction this is (a junction whose tensors hold a row per passage reads it)."""
 
     layer: int
     reads_cache_of: Optional[int] = None
     before: Optional[str] = None
+    passage: int = 0
 
 
 @dataclass(frozen=True)
