@@ -222,8 +222,8 @@ def bogivik_models(size: dict, positions: int):
 
 def design_facts(net):
     """What the roofline of any model of the package needs, read off its plan: the weights of its linears (every matrix
-    but the embedding table), and per layer the sizes of its attention (heads, kv heads, key and value size, window,
-    chunk) and of its matrix memory (heads, key and value size)."""
+    but the embedding table), and per layer of its attention ``(multiply-adds a query spends per key it sees, numbers
+    the cache holds per key, window, chunk, kept first keys)`` and the sizes of its matrix memory (heads, key and value size)."""
     from types import SimpleNamespace
 
     plan = net.plan
@@ -235,7 +235,17 @@ def design_facts(net):
         kind = getattr(spec, "kind", None)
         if kind == "attention":
             dv = spec.head_dim if getattr(spec, "value_dim", None) is None else spec.value_dim
-            attention.append((spec.n_heads, spec.n_kv_heads, spec.head_dim, dv, getattr(spec, "window", None), getattr(spec, "chunk", None)))
+            attention.append((spec.n_heads * (spec.head_dim + dv), spec.n_kv_heads * (spec.head_dim + dv),
+                              getattr(spec, "window", None), getattr(spec, "chunk", None), 0))
+        elif kind == "differential_attention":
+            # two maps per head, each a score and a value product; the cache holds two keys and one value per kv head
+            mask = spec.mask
+            attention.append((2 * spec.n_heads * (spec.head_dim + spec.value_dim), spec.n_kv_heads * (2 * spec.head_dim + spec.value_dim),
+                              mask.size if mask is not None else None, None, mask.keep_first if mask is not None else 0))
+        elif kind == "latent_attention":
+            # per head a score over the plain and the rotated part and a value product; the cache holds the latent and
+            # the shared rotated key part
+            attention.append((spec.n_heads * (spec.head_dim + spec.rot_dim + spec.value_dim), spec.kv_rank + spec.rot_dim, None, None, 0))
         elif kind == "matrix_memory":
             memory.append((spec.n_heads, spec.head_dim, spec.value_dim))
         elif kind == "branches":
@@ -247,21 +257,21 @@ def design_facts(net):
     return SimpleNamespace(linear=linear, attention=attention, memory=memory, width=plan.dim, vocab=plan.vocab_size)
 
 
-def _keys_seen(place: int, window, chunk) -> int:
+def _keys_seen(place: int, window, chunk, keep_first: int = 0) -> int:
     lo = 0
     if window is not None:
         lo = max(lo, place + 1 - window)
     if chunk is not None:
         lo = max(lo, place // chunk * chunk)
-    return place + 1 - lo
+    return place + 1 - lo + min(keep_first, lo)
 
 
 def design_flops(f, tokens: int) -> float:
     """Multiply-adds x 2 of a prompt of ``tokens`` places: the linears (the head at the last place only), score and value
     products over the keys each place sees, the matrix memory's update and read-out (two multiply-adds a number of state)."""
     total = 2.0 * tokens * (f.linear - f.width * f.vocab) + 2.0 * f.width * f.vocab
-    for h, _g, d, dv, window, chunk in f.attention:
-        total += 2.0 * h * (d + dv) * sum(_keys_seen(p, window, chunk) for p in range(tokens))
+    for per_key, _held, window, chunk, kept in f.attention:
+        total += 2.0 * per_key * sum(_keys_seen(p, window, chunk, kept) for p in range(tokens))
     for h, d, dv in f.memory:
         total += 2.0 * 2.0 * h * d * dv * tokens
     return total
@@ -271,15 +281,66 @@ def design_decode_bytes(f, batch: int, context: int, size: int) -> float:
     """Bytes a decode step must move: every weight once, of every row the keys and values it sees, and its matrix
     memories' fp32 state read and written."""
     total = float(size) * f.linear
-    for _h, g, d, dv, window, chunk in f.attention:
-        total += size * batch * g * (d + dv) * _keys_seen(context, window, chunk)
+    for _per_key, held, window, chunk, kept in f.attention:
+        total += size * batch * held * _keys_seen(context, window, chunk, kept)
     for h, d, dv in f.memory:
         total += 2.0 * 4 * batch * h * (d * dv + d + 1)
     return total
 
 
+# Sizes at which Letevik is measured beside the Moondream decoder: width, gated feed-forward (Moondream's plain one gets
+# one and a half times the hidden size: the same weights), the differential layers' heads, kv heads, size of a map and of
+# a value, taps, window and kept keys, the latent layers' heads, plain and rotated key size, value size and the two
+# ranks, the order of layers (d: differential, l: latent) and the looped stretch with its passes. Moondream gets as many
+# layers as Letevik has runs of layers, and heads of the size of a pair of maps. "w2048" has latent rows of 128 numbers
+# (what the matrix-core attention kernel takes), "w4096" rows of 576 (the sizes of latent attention as published
+# models have them; the generic kernel runs).
+LETEVIK_SIZES = {
+    "w2048": dict(width=2048, ff=5632, diff=dict(heads=16, kv_heads=4, dim=64, vdim=128, conv=4, window=1024, keep=4),
+                  latent=dict(heads=16, dim=64, rot_dim=32, vdim=64, q_rank=512, kv_rank=96), order="dlld", loop=(0, 2, 2),
+                  moondream=dict(heads=32, kv_heads=8, head=64)),
+    "w4096": dict(width=4096, ff=7168, diff=dict(heads=16, kv_heads=4, dim=128, vdim=128, conv=4, window=2048, keep=16),
+                  latent=dict(heads=32, dim=128, rot_dim=64, vdim=128, q_rank=1536, kv_rank=512), order="dl", loop=(0, 2, 2),
+                  moondream=dict(heads=32, kv_heads=8, head=128)),
+}
+
+
+def letevik_models(size: dict, positions: int):
+    """``{name: (config dict, registry name)}`` of Letevik and of the Moondream decoder at one size."""
+    w, d, m = size["width"], size["diff"], size["latent"]
+    mlp = {"kind": "dense", "ff": size["ff"], "limit": 7.0}
+    differential = {"heads": d["heads"], "kv_heads": d["kv_heads"], "dim": d["dim"], "vdim": d["vdim"], "scale": d["dim"] ** -0.5,
+                    "diff": 0.5, "conv": d["conv"], "mask": {"size": d["window"], "keep_first": d["keep"]},
+                    "rot": {"base": 10000.0, "dims": d["dim"]}}
+    latent = {"heads": m["heads"], "dim": m["dim"], "rot_dim": m["rot_dim"], "vdim": m["vdim"], "q_rank": m["q_rank"],
+              "kv_rank": m["kv_rank"], "scale": (m["dim"] + m["rot_dim"]) ** -0.5, "rot": {"base": 50000.0, "dims": m["rot_dim"]}}
+    layers = [{"type": "attention", "mixer": dict(differential), "mlp": mlp} if kind == "d" else
+              {"type": "latent_attention", "mixer": dict(latent), "mlp": mlp} for kind in size["order"]]
+    start, stop, times = size["loop"]
+    letevik = {"architecture": "Letevik", "vocab": COMPARE_VOCAB, "width": w, "norm": {"eps": 1e-6}, "max_positions": positions,
+               "embedding": {"bigram": {"buckets": 65521, "mul_prev": 31, "mul_cur": 17}}, "layers": layers,
+               "loop": {"start": start, "stop": stop, "times": times}}
+    md = size["moondream"]
+    runs = len(size["order"]) + (stop - start) * (times - 1)
+    moondream = {"text": {"dim": w, "ff_dim": size["ff"] * 3 // 2, "n_layers": runs, "vocab_size": COMPARE_VOCAB,
+                          "max_context": positions, "n_heads": md["heads"], "n_kv_heads": md["kv_heads"], "head_dim": md["head"],
+                          "rotary_dim": md["head"] // 2, "rope_theta": 10000.0, "prefix_attn": 0, "layer_norm_eps": 1e-5}}
+    return {"letevik": (letevik, "letevik"), "moondream2": (moondream, "moondream2")}
+
+
 def run_compare_bogivik(args, dtype, device) -> dict:
     """Bogivik beside the Moondream decoder at equal sizes, through the same step function."""
+    return run_compare_design(args, dtype, device, "bogivik", BOGIVIK_SIZES, bogivik_models)
+
+
+def run_compare_letevik(args, dtype, device) -> dict:
+    """Letevik beside the Moondream decoder at equal sizes, through the same step function."""
+    return run_compare_design(args, dtype, device, "letevik", LETEVIK_SIZES, letevik_models)
+
+
+def run_compare_design(args, dtype, device, design: str, sizes: dict, models) -> dict:
+    """A design beside the Moondream decoder at the sizes of ``sizes`` (``models(size, positions)`` gives both configurations),
+    through the same step function."""
     from types import SimpleNamespace
 
     import torch
@@ -287,11 +348,11 @@ def run_compare_bogivik(args, dtype, device) -> dict:
     size_bytes = 2 if dtype == torch.bfloat16 else 4
     context, tokens = args.context, args.prefill_tokens
     positions = max(context + args.steps + args.warmup + 16, tokens)
-    labels = (args.compare_sizes or ",".join(BOGIVIK_SIZES)).split(",")
+    labels = (args.compare_sizes or ",".join(sizes)).split(",")
     out = {}
     for label in labels:
         out[label] = {}
-        for name, (config, registry_name) in bogivik_models(BOGIVIK_SIZES[label], positions).items():
+        for name, (config, registry_name) in models(sizes[label], positions).items():
             if args.compare_model not in ("both", name):
                 continue
             net, _typed = build_from_config(config, registry_name, dtype, device)
@@ -313,13 +374,13 @@ def run_compare_bogivik(args, dtype, device) -> dict:
             del net
             torch.cuda.empty_cache()
     first = out[labels[0]]
-    lead = first.get("bogivik") or next(iter(first.values()))
+    lead = first.get(design) or next(iter(first.values()))
     key = "decode_b8" if "decode_b8" in lead else next((k for k in lead if k.startswith("decode")), None)
-    return {"metric": f"Bogivik beside the Moondream decoder at equal sizes: decode tok/s at batch 8, context {context} ({labels[0]})",
+    return {"metric": f"{design.capitalize()} beside the Moondream decoder at equal sizes: decode tok/s at batch 8, context {context} ({labels[0]})",
             "value": lead[key]["tok_s"] if key else None, "unit": "tok/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
             "ms_per_step": lead[key]["ms_per_step"] if key else None, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
             "dtype": args.dtype, "data": "synthetic (seeded random token ids, random weights N(0,0.02))",
-            "config": {"model": "bogivik and moondream2-text at equal sizes", "sizes": {k: BOGIVIK_SIZES[k] for k in out},
+            "config": {"model": f"{design} and moondream2-text at equal sizes", "sizes": {k: sizes[k] for k in out},
                        "global_batch": 8, "seq_len": context, "vocab_size": COMPARE_VOCAB, "parallelism": "single-gpu"},
             "compare": out}
 
@@ -611,16 +672,17 @@ def main() -> int:
                         help="with --workload: RuntimeConfig.tune_linears (time the vendor library's algorithms at warm-up)")
     parser.add_argument("--check", type=int, default=0,
                         help="with --workload: compare this many greedy requests with the plain implementation (for --layers 2)")
-    parser.add_argument("--workload", default="decode", choices=["decode", "waves256", "mixed48", "compare-vimesun", "compare-bogivik"],
+    parser.add_argument("--workload", default="decode", choices=["decode", "waves256", "mixed48", "compare-vimesun", "compare-bogivik", "compare-letevik"],
                         help="decode: the benchmark's decode step (default); waves256 and mixed48 run requests through "
-                             "InferenceEngine; compare-vimesun and compare-bogivik measure that design beside the Moondream decoder at equal sizes")
+                             "InferenceEngine; compare-vimesun, compare-bogivik and compare-letevik measure that design beside the Moondream "
+                             "decoder at equal sizes")
     parser.add_argument("--compare-sizes", default=None,
-                        help="with --workload compare-vimesun or compare-bogivik: which of its sizes, with commas between them "
+                        help="with --workload compare-*: which of its sizes, with commas between them "
                              "(default: all of them)")
-    parser.add_argument("--compare-model", default="both", choices=["both", "vimesun", "bogivik", "moondream2"],
+    parser.add_argument("--compare-model", default="both", choices=["both", "vimesun", "bogivik", "letevik", "moondream2"],
                         help="with --workload compare-*: one of the two designs only (for profiling)")
-    parser.add_argument("--compare-batches", default="1,8,64", help="with --workload compare-bogivik: batch sizes of the decode steps")
-    parser.add_argument("--skip-prefill", action="store_true", help="with --workload compare-bogivik: decode steps only")
+    parser.add_argument("--compare-batches", default="1,8,64", help="with --workload compare-bogivik or compare-letevik: batch sizes of the decode steps")
+    parser.add_argument("--skip-prefill", action="store_true", help="with --workload compare-bogivik or compare-letevik: decode steps only")
     parser.add_argument("--max-batch-size", type=int, default=None, help="for the workloads through the entry point")
     parser.add_argument("--linears", default="library", choices=["library", "own"],
                         help="linears of more than 64 rows (a prompt's): through hipBLASLt (the engine's default) or "
@@ -652,6 +714,9 @@ def main() -> int:
         return 0
     if args.workload == "compare-bogivik":
         print(json.dumps(run_compare_bogivik(args, dtype, device)))
+        return 0
+    if args.workload == "compare-letevik":
+        print(json.dumps(run_compare_letevik(args, dtype, device)))
         return 0
     if args.workload != "decode":
         print(json.dumps(run_workload(args, dict(SIZES[args.sizes]))))

@@ -13,6 +13,17 @@
 // and the weights are exp(s_j) / (sum_j exp(s_j) [+ exp(sink)]): fp32 throughout; the weights enter
 // the value product as bf16, sums in fp32.
 //
+// Further forms of the same loop, for mixers that are attention with a twist:
+//  * sinks (fp32 [H]): the valueless term's score per head instead of one number;
+//  * keep_first: a query also sees the keys [0, min(keep_first, kv_lo)) of its row, before its window
+//    (their tiles are taken ahead of the window's);
+//  * maps > 1: query and key heads come in groups of `maps` neighbours, map m of a query head reads map m of
+//    its key head, and all maps of a key head share one value head (H and Hkv count maps, the value cache has
+//    Hkv / maps heads);
+//  * values_in_keys: a key's value is the first hdv channels of its key row (a cache of latents that are keys
+//    and values at once); the value operand is then gathered from the key page;
+//  * out_f32: outputs leave as fp32.
+//
 // A workgroup owns 32 columns of the score product and one kv head. In a step with prompt portions a
 // column is a query of a block of 32 consecutive tokens of one row and one query head (the host lists the
 // blocks); in a decode step, where every row has one token, the columns are the query heads that share the
@@ -60,7 +71,8 @@ attn_biased_kernel(const bf16_t* __restrict__ q, long q_row_stride, const bf16_t
                    const int* __restrict__ positions, const float* __restrict__ slopes, bf16_t* __restrict__ out,
                    long out_row_stride, float scale, int H, int Hkv, int hdv, int heads_per_block, int has_sink,
                    float sink_score, const float* __restrict__ bias_table, int bias_len, const bf16_t* __restrict__ gate,
-                   long gate_row_stride) {
+                   long gate_row_stride, const float* __restrict__ sinks, int keep_first, int maps, int values_in_keys,
+                   int out_f32) {
     constexpr int HD = NK * 16;
     constexpr int REC = 16 * NV + 2;            // floats a lane hands over at a merge: its outputs, m and l
     extern __shared__ float mrg[];              // [waves / 2][REC][64]
@@ -75,12 +87,13 @@ attn_biased_kernel(const bf16_t* __restrict__ q, long q_row_stride, const bf16_t
         kvh = blockIdx.x / groups;
         const int hq = (blockIdx.x % groups) * heads_per_block + col;
         live = col < heads_per_block && hq < G;
-        head = kvh * G + (live ? hq : 0);
+        // (maps == 1: head kvh * G + hq)
+        head = ((kvh / maps) * G + (live ? hq : 0)) * maps + kvh % maps;
         tok = blockIdx.y;
         row = token_row[tok];
     } else {
         head = blockIdx.x;
-        kvh = head / G;
+        kvh = (head / maps / G) * maps + head % maps;
         const int blk = blockIdx.y;
         row = qblk_row[blk];
         const int tok_end = cu_q[row + 1];
@@ -113,7 +126,8 @@ attn_biased_kernel(const bf16_t* __restrict__ q, long q_row_stride, const bf16_t
     const int place = (slopes || bias_table) ? positions[tok] : 0;
     const float* bias_row = bias_table ? bias_table + (size_t)head * bias_len : nullptr;
     const float bias_far2 = bias_row ? bias_row[bias_len - 1] * AB_LOG2E : 0.f;
-    const float sink2 = sink_score * AB_LOG2E;
+    const float sink2 = (sinks ? sinks[head] : sink_score) * AB_LOG2E;
+    const int vh = kvh / maps, Hv = Hkv / maps;
 
     float m = has_sink ? sink2 : -INFINITY;     // reference point of this lane's column (the same in both halves)
     float l = 0.f;                              // this lane's share of the column's sum
@@ -128,7 +142,7 @@ attn_biased_kernel(const bf16_t* __restrict__ q, long q_row_stride, const bf16_t
     const int krow = (col & 0x13) | ((col & 4) << 1) | ((col & 8) >> 1);
     const int kpage_in_tile = krow >> 4, kslot = krow & 15;
     const size_t k_head = (size_t)kvh * AB_PAGE * HD, k_page = (size_t)Hkv * AB_PAGE * HD;
-    const size_t v_page = (size_t)Hkv * hdv * AB_PAGE;
+    const size_t v_page = (size_t)Hv * hdv * AB_PAGE;
     // the value rows (channels) this lane loads: clamped into the head where the last block is not full
     int vch[NV];
 #pragma unroll
@@ -136,7 +150,11 @@ attn_biased_kernel(const bf16_t* __restrict__ q, long q_row_stride, const bf16_t
 
     if (blk_lo < blk_hi) {
         const int first_tile = blk_lo / AB_TILE, last_tile = (blk_hi - 1) / AB_TILE;
-        for (int tile = first_tile + wave; tile <= last_tile; tile += n_waves) {
+        // tiles of kept first keys that lie wholly before the window's first tile come ahead of the window's
+        const int kept_tiles = min((min(keep_first, blk_lo) + AB_TILE - 1) / AB_TILE, first_tile);
+        const int n_tiles = kept_tiles + last_tile - first_tile + 1;
+        for (int turn = wave; turn < n_tiles; turn += n_waves) {
+            const int tile = turn < kept_tiles ? turn : first_tile + (turn - kept_tiles);
             const int base = tile * AB_TILE;
             // pages of the tile (a page the row has given back, or none: any page, its keys are masked)
             int pg[2];
@@ -152,12 +170,24 @@ attn_biased_kernel(const bf16_t* __restrict__ q, long q_row_stride, const bf16_t
                 for (int c = 0; c < NK; ++c) kr[c] = *reinterpret_cast<const ab_bf16x8*>(kp + c * 16);
             }
             ab_bf16x8 vr[2][NV];
+            if (values_in_keys) {
+                // eight consecutive keys of one channel: a column of the row-major key page
 #pragma unroll
-            for (int p = 0; p < 2; ++p)
+                for (int p = 0; p < 2; ++p) {
+                    const bf16_t* vp = k_cache + (size_t)pg[p] * k_page + k_head + (size_t)(half * 8) * HD;
 #pragma unroll
-                for (int b = 0; b < NV; ++b)
-                    vr[p][b] = *reinterpret_cast<const ab_bf16x8*>(v_cache + (size_t)pg[p] * v_page +
-                                                                   ((size_t)kvh * hdv + vch[b]) * AB_PAGE + half * 8);
+                    for (int b = 0; b < NV; ++b)
+#pragma unroll
+                        for (int e = 0; e < 8; ++e) vr[p][b][e] = vp[(size_t)e * HD + vch[b]];
+                }
+            } else {
+#pragma unroll
+                for (int p = 0; p < 2; ++p)
+#pragma unroll
+                    for (int b = 0; b < NV; ++b)
+                        vr[p][b] = *reinterpret_cast<const ab_bf16x8*>(v_cache + (size_t)pg[p] * v_page +
+                                                                       ((size_t)vh * hdv + vch[b]) * AB_PAGE + half * 8);
+            }
             ab_floatx16 s;
 #pragma unroll
             for (int i = 0; i < 16; ++i) s[i] = 0.f;
@@ -166,7 +196,7 @@ attn_biased_kernel(const bf16_t* __restrict__ q, long q_row_stride, const bf16_t
             // register i of this lane: key base + (i / 8) * 16 + half * 8 + i % 8 of the lane's column
             const int j0 = base + half * 8;
             const float bias0 = -slope2 * (float)(place - j0);          // (an integer distance: exact)
-            const bool whole = base >= max_lo && base + AB_TILE <= min_hi;
+            const bool whole = turn >= kept_tiles && base >= max_lo && base + AB_TILE <= min_hi;
             if (!whole) {
                 // Keys that no column of the block sees (slots behind the row's last key, pages given back) may hold
                 // anything, a NaN included, and a weight of 0 does not clear that in a product: their values are zeroed.
@@ -175,7 +205,7 @@ attn_biased_kernel(const bf16_t* __restrict__ q, long q_row_stride, const bf16_t
 #pragma unroll
                     for (int e = 0; e < 8; ++e) {
                         const int j = base + p * AB_PAGE + half * 8 + e;
-                        if (j < blk_lo || j >= blk_hi) {
+                        if ((j < blk_lo && j >= keep_first) || j >= blk_hi) {
 #pragma unroll
                             for (int b = 0; b < NV; ++b) vr[p][b][e] = (bf16_t)0.f;
                         }
@@ -193,7 +223,7 @@ attn_biased_kernel(const bf16_t* __restrict__ q, long q_row_stride, const bf16_t
                 else x += bias_far2;
                 if (!whole) {
                     const int j = j0 + off;
-                    if (j < lo || j >= hi) x = -INFINITY;
+                    if ((j < lo && j >= keep_first) || j >= hi) x = -INFINITY;
                 }
                 s[i] = x;
                 tile_max = fmaxf(tile_max, x);
@@ -267,7 +297,8 @@ attn_biased_kernel(const bf16_t* __restrict__ q, long q_row_stride, const bf16_t
     }
     const float inv = l > 0.f ? 1.0f / l : 0.f;
     // register i of block b: channel b * 32 + (i / 4) * 8 + half * 4 + i % 4 of the lane's column
-    bf16_t* op = out + (size_t)tok * out_row_stride + (size_t)head * hdv;
+    const size_t out_at = (size_t)tok * out_row_stride + (size_t)head * hdv;
+    bf16_t* op = out + out_at;
     if (gate) {
         // an output gate: every channel times the sigmoid of the gate's pre-activation of the same token and channel
         const bf16_t* gp = gate + (size_t)tok * gate_row_stride + (size_t)head * hdv;
@@ -278,6 +309,24 @@ attn_biased_kernel(const bf16_t* __restrict__ q, long q_row_stride, const bf16_t
                 const int ch = b * 32 + (i / 4) * 8 + half * 4 + i % 4;
                 if (ch < hdv) o[b][i] *= 1.0f / (1.0f + __expf(-(float)gp[ch]));
             }
+    }
+    if (out_f32) {
+        float* fp = reinterpret_cast<float*>(out) + out_at;
+#pragma unroll
+        for (int b = 0; b < NV; ++b)
+#pragma unroll
+            for (int g4 = 0; g4 < 4; ++g4) {
+                const int ch = b * 32 + g4 * 8 + half * 4;
+                if (ch + 3 < hdv) {
+                    float4 y = make_float4(o[b][g4 * 4] * inv, o[b][g4 * 4 + 1] * inv, o[b][g4 * 4 + 2] * inv, o[b][g4 * 4 + 3] * inv);
+                    *reinterpret_cast<float4*>(fp + ch) = y;
+                } else {
+#pragma unroll
+                    for (int e = 0; e < 4; ++e)
+                        if (ch + e < hdv) fp[ch + e] = o[b][g4 * 4 + e] * inv;
+                }
+            }
+        return;
     }
 #pragma unroll
     for (int b = 0; b < NV; ++b)
@@ -299,10 +348,10 @@ attn_biased_kernel(const bf16_t* __restrict__ q, long q_row_stride, const bf16_t
 
 static bool ab_sizes_covered(int hd, int hdv) {
     const int nk = hd / 16, nv = (hdv + 31) / 32;
-    return hd % 16 == 0 && hdv % 4 == 0 && (nk == 2 || nk == 3 || nk == 4 || nk == 6 || nk == 8) && nv >= 1 && nv <= 4;
+    return hd % 16 == 0 && hdv % 4 == 0 && nk >= 2 && nk <= 8 && nv >= 1 && nv <= 4;
 }
 
-// Whether the kernel covers these sizes: query/key heads of 32, 48, 64, 96 or 128 channels, value heads of up to
+// Whether the kernel covers these sizes: query/key heads of 32 to 128 channels in steps of 16, value heads of up to
 // 128 in steps of 4, pages of 16.
 KA_API int ka_attention_biased_supported(int hd, int hdv, int page_size) {
     return page_size == AB_PAGE && ab_sizes_covered(hd, hdv) ? 1 : 0;
@@ -318,15 +367,21 @@ KA_API int ka_attention_biased_bf16(const void* q, long q_row_stride, const void
                                     const int* kv_hi, const int* positions, const float* slopes, void* out,
                                     long out_row_stride, float scale, int n, int H, int Hkv, int hd, int hdv,
                                     int page_size, int waves, int has_sink, float sink_score, const float* bias_table,
-                                    int bias_len, const void* gate, long gate_row_stride, hipStream_t stream) {
+                                    int bias_len, const void* gate, long gate_row_stride, const float* sinks, int keep_first,
+                                    int maps, int values_in_keys, int out_f32, hipStream_t stream) {
     const char* who = "ka_attention_biased_bf16";
     KA_CHECK(n >= 0 && n_blocks >= 0 && H > 0 && Hkv > 0 && H % Hkv == 0, "%s: bad sizes", who);
     KA_CHECK(page_size == AB_PAGE && ab_sizes_covered(hd, hdv), "%s: head sizes %d / %d or page size %d not covered", who, hd, hdv, page_size);
     KA_CHECK(max_pages > 0, "%s: bad table width %d", who, max_pages);
     KA_CHECK(waves == 4 || waves == 8, "%s: %d waves", who, waves);
-    KA_CHECK((uintptr_t)q % 16 == 0 && q_row_stride % 8 == 0 && (uintptr_t)k_cache % 16 == 0 && (uintptr_t)v_cache % 16 == 0,
+    KA_CHECK((uintptr_t)q % 16 == 0 && q_row_stride % 8 == 0 && (uintptr_t)k_cache % 16 == 0,
              "%s: operands must be 16-byte aligned", who);
-    KA_CHECK((uintptr_t)out % 8 == 0 && out_row_stride % 4 == 0, "%s: output rows must be 8-byte aligned", who);
+    KA_CHECK((uintptr_t)out % (out_f32 ? 16 : 8) == 0 && out_row_stride % 4 == 0, "%s: output rows must be aligned to four values", who);
+    KA_CHECK(maps >= 1 && H % maps == 0 && Hkv % maps == 0 && keep_first >= 0, "%s: %d maps do not divide the heads %d and %d", who, maps, H, Hkv);
+    KA_CHECK(!values_in_keys || (hdv <= hd && maps == 1), "%s: values inside keys of %d channels cannot have %d", who, hd, hdv);
+    KA_CHECK(sinks == nullptr || has_sink, "%s: sink scores without a sink", who);
+    KA_CHECK(!out_f32 || gate == nullptr, "%s: the output gate goes with bf16 outputs", who);
+    KA_CHECK(values_in_keys || (uintptr_t)v_cache % 16 == 0, "%s: operands must be 16-byte aligned", who);
     KA_CHECK(slopes == nullptr || positions != nullptr, "%s: slopes need the queries' positions", who);
     KA_CHECK(bias_table == nullptr || (positions != nullptr && bias_len > 0), "%s: a distance table needs the queries' positions", who);
     KA_CHECK(n_blocks == 0 || (qblk_row && qblk_tok && cu_q), "%s: blocks of queries need their lists", who);
@@ -356,10 +411,10 @@ KA_API int ka_attention_biased_bf16(const void* q, long q_row_stride, const void
                            q_row_stride, (const bf16_t*)k_cache, (const bf16_t*)v_cache, block_table, max_pages, qblk_row, \
                            qblk_tok, cu_q, token_row, kv_lo, kv_hi, positions, slopes, (bf16_t*)out, out_row_stride, scale, \
                            H, Hkv, hdv, heads_per_block, has_sink, sink_score, bias_table, bias_len, (const bf16_t*)gate, \
-                           gate_row_stride);                                                                               \
+                           gate_row_stride, sinks, keep_first, maps, values_in_keys, out_f32);                                                                            \
     }
 #define AB_LAUNCH_NK(NK) AB_LAUNCH(NK, 1) AB_LAUNCH(NK, 2) AB_LAUNCH(NK, 3) AB_LAUNCH(NK, 4)
-    AB_LAUNCH_NK(2) AB_LAUNCH_NK(3) AB_LAUNCH_NK(4) AB_LAUNCH_NK(6) AB_LAUNCH_NK(8)
+    AB_LAUNCH_NK(2) AB_LAUNCH_NK(3) AB_LAUNCH_NK(4) AB_LAUNCH_NK(5) AB_LAUNCH_NK(6) AB_LAUNCH_NK(7) AB_LAUNCH_NK(8)
 #undef AB_LAUNCH_NK
 #undef AB_LAUNCH
     KA_LAUNCH_CHECK();

@@ -57,7 +57,8 @@ _SIGNATURES = {
         _c_void_p, _c_long, _c_void_p, _c_void_p, _c_int, _c_long, _c_int, _c_int, _c_void_p],      # W, ldw, bias, out, ..., stream
     "ka_attention_biased_bf16": [_c_void_p, _c_long, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_void_p, _c_void_p, _c_int,
                                  _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_long, _c_float,
-                                 _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_void_p, _c_int, _c_void_p, _c_long, _c_void_p],
+                                 _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_void_p, _c_int, _c_void_p, _c_long,
+                                 _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_void_p],
     "ka_matrix_memory_chunks_bf16": [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_long, _c_void_p, _c_void_p, _c_void_p, _c_void_p,
                                      _c_void_p, _c_void_p, _c_long, _c_int, _c_int, _c_int, _c_int, _c_float, _c_float, _c_float,
                                      _c_void_p, _c_int, _c_void_p],
@@ -616,11 +617,14 @@ def biased_query_block(head_dim: int, value_dim: int) -> Optional[int]:
 
 
 def attention_biased_bf16(q, k_cache, v_cache, block_table, token_row, kv_lo, kv_hi, out, scale, n_heads, n_kv_heads,
-                          head_dim, value_dim, positions, slopes, sink, batch, bias_table=None, gate=None) -> bool:
+                          head_dim, value_dim, positions, slopes, sink, batch, bias_table=None, gate=None, sinks=None,
+                          keep_first: int = 0, maps: int = 1, values_in_keys: bool = False) -> bool:
     """Attention with the further terms of ``ops.core.attention_generic`` (values of ``value_dim`` channels, ``slopes``
-    times the distance taken off the scores, a ``sink`` in the softmax's denominator) on the matrix cores, for prompt
-    portions, mixed steps and decode steps alike. False: not covered (head sizes, page size, alignment, no list of
-    blocks of 32 queries with the step), nothing was run."""
+    times the distance taken off the scores, a ``sink`` in the softmax's denominator or one per head in ``sinks``, kept
+    first keys before the window, several maps per head over shared values, values that are the first channels of the
+    keys, fp32 outputs where ``out`` is fp32) on the matrix cores, for prompt portions, mixed steps and decode steps
+    alike. False: not covered (head sizes, page size, alignment, no list of blocks of 32 queries with the step),
+    nothing was run."""
     n = q.shape[0]
     page_size = k_cache.shape[2]
     if n == 0:
@@ -628,9 +632,16 @@ def attention_biased_bf16(q, k_cache, v_cache, block_table, token_row, kv_lo, kv
     handle = lib()
     if batch is None or not handle.ka_attention_biased_supported(int(head_dim), int(value_dim), int(page_size)):
         return False
-    if q.dtype != torch.bfloat16 or q.data_ptr() % 16 or q.stride(0) % 8 or q.stride(1) != 1 or out.data_ptr() % 8 \
-            or out.stride(0) % 4 or out.stride(1) != 1 or k_cache.data_ptr() % 16 or v_cache.data_ptr() % 16:
+    out_f32 = out.dtype == torch.float32
+    if q.dtype != torch.bfloat16 or q.data_ptr() % 16 or q.stride(0) % 8 or q.stride(1) != 1 or out.data_ptr() % (16 if out_f32 else 8) \
+            or out.stride(0) % 4 or out.stride(1) != 1 or k_cache.data_ptr() % 16 or (v_cache is not None and v_cache.data_ptr() % 16):
         return False
+    if (v_cache is None) != bool(values_in_keys) or (values_in_keys and (maps != 1 or value_dim > head_dim)) or (out_f32 and gate is not None):
+        return False
+    if n_heads % maps or n_kv_heads % maps:
+        raise KernelError("attention: the maps must divide the heads")
+    if sinks is not None and (sinks.dtype != torch.float32 or sinks.numel() != n_heads or not sinks.is_contiguous()):
+        raise KernelError("attention: sink scores must be fp32 [H]")
     if slopes is not None and (slopes.dtype != torch.float32 or slopes.numel() != n_heads or positions is None):
         raise KernelError("attention: slopes must be fp32 [H] and come with the queries' positions")
     if gate is not None and (gate.dtype != torch.bfloat16 or gate.dim() != 2 or gate.stride(1) != 1
@@ -658,13 +669,29 @@ def attention_biased_bf16(q, k_cache, v_cache, block_table, token_row, kv_lo, kv
     if n > 65535:
         return False
     _check(handle.ka_attention_biased_bf16(
-        q.data_ptr(), q.stride(0), k_cache.data_ptr(), v_cache.data_ptr(), block_table.data_ptr(), block_table.shape[1],
+        q.data_ptr(), q.stride(0), k_cache.data_ptr(), _ptr(v_cache), block_table.data_ptr(), block_table.shape[1],
         _ptr(rows), _ptr(first), n_blocks, batch.cu_q.data_ptr(), token_row.data_ptr(), _ptr(kv_lo), kv_hi.data_ptr(),
         _ptr(positions), _ptr(slopes), out.data_ptr(), out.stride(0), float(scale), n, n_heads, n_kv_heads, head_dim,
-        value_dim, page_size, waves, int(sink is not None), float(sink or 0.0), _ptr(bias_table),
+        value_dim, page_size, waves, int(sink is not None or sinks is not None), float(sink or 0.0), _ptr(bias_table),
         int(bias_table.shape[1]) if bias_table is not None else 0, _ptr(gate),
-        (gate.stride(0) if n > 1 else n_heads * value_dim) if gate is not None else 0, stream_ptr()))
+        (gate.stride(0) if n > 1 else n_heads * value_dim) if gate is not None else 0, _ptr(sinks), int(keep_first), int(maps),
+        int(bool(values_in_keys)), int(out_f32), stream_ptr()))
     return True
+
+
+def attention_maps_bf16(q, k_cache, v_cache, block_table, token_row, kv_lo, kv_hi, out, scale, n_heads, n_kv_heads, head_dim,
+                        value_dim, keep_first, maps, batch) -> bool:
+    """``maps`` attentions per head over shared values behind a window that keeps the first keys (``n_heads`` and
+    ``n_kv_heads`` count maps), outputs in fp32 ``[n, n_heads value_dim]``, on the matrix cores. False: not covered."""
+    return attention_biased_bf16(q, k_cache, v_cache, block_table, token_row, kv_lo, kv_hi, out, scale, n_heads, n_kv_heads,
+                                 head_dim, value_dim, None, None, None, batch, keep_first=keep_first, maps=maps)
+
+
+def attention_latent_bf16(q, cache, block_table, token_row, kv_hi, out, scale, n_heads, row_dim, rank, sinks, batch) -> bool:
+    """``n_heads`` query heads of ``row_dim`` channels over one cached row per key whose first ``rank`` channels are its
+    value, with a sink score per head, on the matrix cores. False: not covered (rows above 128 channels among others)."""
+    return attention_biased_bf16(q, cache, None, block_table, token_row, None, kv_hi, out, scale, n_heads, 1, row_dim, rank,
+                                 None, None, None, batch, sinks=sinks, values_in_keys=True)
 
 
 def matrix_memory_chunks_scratch(n: int, n_rows: int, n_heads: int, head_dim: int, value_dim: int) -> int:

@@ -93,6 +93,12 @@ class DifferentialAttention(Mixer):
                 raise ValueError(f"differential attention cannot apply this rotation to heads of {spec.head_dim} channels")
             self._freqs, self._pairing = rotation.frequencies.to(device).contiguous(), rotation.pairing
 
+    def query_tile(self) -> Optional[int]:
+        if self.dtype != torch.bfloat16:
+            return None                     # the generic kernel takes tokens one by one
+        from ..ops import fast
+        return fast.biased_query_block(self.spec.head_dim, self.spec.value_dim)
+
     def input_projection(self):
         return None        # (the block runs this mixer through ``forward``)
 

@@ -85,6 +85,12 @@ class LatentAttention(Mixer):
                 raise ValueError(f"latent attention cannot apply this rotation to a part of {spec.rot_dim} channels")
             self._freqs, self._pairing = rotation.frequencies.to(device).contiguous(), rotation.pairing
 
+    def query_tile(self) -> Optional[int]:
+        if self.dtype != torch.bfloat16:
+            return None                     # the generic kernel takes tokens one by one
+        from ..ops import fast
+        return fast.biased_query_block(self.row_dim, self.spec.kv_rank)
+
     def attend(self, down, batch, cache: LayerCache, beside=None) -> torch.Tensor:
         """From the projected row ``[c_q' | c' | k_r | gate]`` to the gated heads, the input of the output projection."""
         spec = self.spec

@@ -2,6 +2,7 @@
 implementation, under every way of cutting the work; and each of its mechanisms' kernels alone."""
 
 import json
+import math
 import os
 import subprocess
 
@@ -614,3 +615,154 @@ def test_latent_rows_kernels(dtype):
     tails = plain.rotate_halves(tails, dr, base)[places]
     got = dst.double().cpu().view(n, H, rank + dr)
     assert torch.allclose(got[:, :, rank:], tails, **tol) and float(got[:, :, :rank].abs().max()) == 0.0
+
+
+# ------------------------------------------------------------------------------------------------ the matrix-core attention's further forms
+class _Packed:
+    """Rows of keys in a paged cache with shuffled pages, and the packed queries of a step over them: row ``r`` has
+    ``lengths[r]`` keys, of which the last ``lengths[r] - starts[r]`` places are this step's queries. Pages that a window
+    has passed and that hold no kept key are given back (the table says -1 and the page holds NaN)."""
+
+    def __init__(self, lengths, starts, window, kept, seed):
+        from types import SimpleNamespace
+
+        self.lengths, self.starts, self.window, self.kept = lengths, starts, window, kept
+        gen = torch.Generator().manual_seed(seed)
+        self.gen = gen
+        n_pages = sum(-(-n // 16) for n in lengths) + 3
+        order = torch.randperm(n_pages, generator=gen).tolist()
+        self.n_pages = n_pages
+        table = torch.full((len(lengths), max(-(-n // 16) for n in lengths) + 1), -1, dtype=torch.int32)
+        for r, n in enumerate(lengths):
+            for p in range(-(-n // 16)):
+                table[r, p] = order.pop()
+        self.full_table = table.clone()
+        if window is not None:
+            for r, s in enumerate(starts):
+                for p in range(max(0, s + 1 - window) // 16):
+                    if p * 16 >= kept:
+                        table[r, p] = -1
+        token_row, kv_lo, kv_hi, cu_q, rows, first = [], [], [], [0], [], []
+        for r, (n, s) in enumerate(zip(lengths, starts)):
+            for b in range(0, n - s, 32):
+                rows.append(r)
+                first.append(len(token_row) + b)
+            for p in range(s, n):
+                token_row.append(r)
+                kv_hi.append(p + 1)
+                kv_lo.append(0 if window is None else max(0, p + 1 - window))
+            cu_q.append(len(token_row))
+        self.n = len(token_row)
+        self.token_row, self.kv_hi, self.cu_q = _i32(token_row), _i32(kv_hi), _i32(cu_q)
+        self.kv_lo = _i32(kv_lo) if window is not None else None
+        self.table = table.to(DEV)
+        self.batch = SimpleNamespace(decode_only=all(n - s == 1 for n, s in zip(lengths, starts)),
+                                     query_blocks={32: (_i32(rows), _i32(first))}, cu_q=self.cu_q)
+
+    def pages(self, per_row, transposed=False):
+        """``per_row[r]`` ``[length, heads, channels]`` into pages ``[pages, heads, 16, channels]`` (or ``[pages, heads, channels, 16]``);
+        pages given back hold NaN."""
+        heads, channels = per_row[0].shape[1:]
+        out = torch.full((self.n_pages, heads, 16, channels), float("nan"), dtype=per_row[0].dtype)
+        for r, rows in enumerate(per_row):
+            for p in range(-(-rows.shape[0] // 16)):
+                if self.table[r, p] >= 0:
+                    part = rows[p * 16:(p + 1) * 16]
+                    out[self.full_table[r, p], :, :part.shape[0]] = part.transpose(0, 1)
+        return (out.transpose(2, 3) if transposed else out).contiguous().to(DEV)
+
+
+_CUTS = {"mixed": ([70, 133, 9, 2, 101, 64, 300], [0, 100, 7, 0, 100, 63, 267]), "decode": ([70, 133, 9, 1, 300], [69, 132, 8, 0, 299])}
+
+
+@pytest.mark.parametrize("cut", list(_CUTS))
+@pytest.mark.parametrize("window, kept", [(24, 4), (40, 0), (7, 9), (33, 17), (64, 40), (None, 0)])
+@pytest.mark.parametrize("hd, hdv", [(32, 64), (64, 32), (48, 20), (128, 128), (80, 96)])
+def test_two_maps_on_the_matrix_cores(hd, hdv, window, kept, cut):
+    """The bf16 kernel for prompts, portions and single tokens: two maps per head over shared values, a window that keeps
+    the first keys whose other pages were given back, fp32 outputs."""
+    from kestrel_amd.ops import fast
+
+    lengths, starts = _CUTS[cut]
+    case = _Packed(lengths, starts, window, kept, seed=hd + hdv)
+    H, G, scale = 4, 2, 1.7 / math.sqrt(hd)
+    bf = torch.bfloat16
+    k = [torch.randn(n, 2 * G, hd, generator=case.gen).to(bf) for n in lengths]
+    v = [torch.randn(n, G, hdv, generator=case.gen).to(bf) for n in lengths]
+    q = [torch.randn(n - s, 2 * H, hd, generator=case.gen).to(bf) for n, s in zip(lengths, starts)]
+    out = torch.full((case.n, 2 * H * hdv), float("nan"), dtype=torch.float32, device=DEV)
+    done = fast.attention_maps_bf16(torch.cat(q).reshape(case.n, -1).to(DEV), case.pages(k), case.pages(v, transposed=True), case.table,
+                                    case.token_row, case.kv_lo, case.kv_hi, out, scale, 2 * H, 2 * G, hd, hdv, kept, 2, case.batch)
+    assert done, "the matrix-core kernel declined sizes it is meant to take"
+    want = []
+    for r, (n, s) in enumerate(zip(lengths, starts)):
+        seen = plain.visible(n, window, kept)[s:]
+        rows = torch.zeros(n - s, 2 * H, hdv, dtype=F64)
+        for head in range(2 * H):
+            which, g = head % 2, head // 2 // (H // G)
+            scores = (q[r].double()[:, head] @ k[r].double()[:, 2 * g + which].T) * scale
+            rows[:, head] = plain.softmax_weights(scores[None], seen)[0] @ v[r].double()[:, g]
+        want.append(rows.reshape(n - s, -1))
+    got, want = out.double().cpu(), torch.cat(want)
+    err = (got - want).abs()
+    assert bool((err <= 3e-2 + 2e-2 * want.abs()).all()), f"max error {float(err.max()):.3g}"
+
+
+@pytest.mark.parametrize("cut", list(_CUTS))
+@pytest.mark.parametrize("heads", [5, 40])
+@pytest.mark.parametrize("rank, dr", [(64, 16), (96, 16), (48, 32), (96, 32), (20, 12)])
+def test_latents_with_sinks_on_the_matrix_cores(rank, dr, heads, cut):
+    """The bf16 kernel over cached rows that are key and value at once, a sink score per head; in a decode step more heads
+    than one workgroup's columns."""
+    from kestrel_amd.ops import fast
+
+    lengths, starts = _CUTS[cut]
+    case = _Packed(lengths, starts, None, 0, seed=rank + dr + heads)
+    scale = 1.5 / math.sqrt(rank + dr)
+    bf = torch.bfloat16
+    rows = [torch.randn(n, 1, rank + dr, generator=case.gen).to(bf) for n in lengths]
+    q = [torch.randn(n - s, heads, rank + dr, generator=case.gen).to(bf) for n, s in zip(lengths, starts)]
+    sinks = torch.linspace(-4.0, 6.0, heads)
+    out = torch.full((case.n, heads * rank), float("nan"), dtype=bf, device=DEV)
+    done = fast.attention_latent_bf16(torch.cat(q).reshape(case.n, -1).to(DEV), case.pages(rows), case.table, case.token_row, case.kv_hi,
+                                      out, scale, heads, rank + dr, rank, sinks.to(DEV), case.batch)
+    assert done, "the matrix-core kernel declined sizes it is meant to take"
+    want = []
+    for r, (n, s) in enumerate(zip(lengths, starts)):
+        c = rows[r].double()[:, 0]
+        scores = torch.einsum("ihd,jd->hij", q[r].double(), c) * scale
+        weights = plain.softmax_weights(scores, plain.visible(n)[s:], sinks.double())
+        want.append(torch.einsum("hij,jd->ihd", weights, c[:, :rank]).reshape(n - s, -1))
+    got, want = out.double().cpu(), torch.cat(want)
+    err = (got - want).abs()
+    assert bool((err <= 3e-2 + 2e-2 * want.abs()).all()), f"max error {float(err.max()):.3g}"
+
+
+def test_the_matrix_core_kernels_run_where_sizes_allow():
+    """In bf16 the model whose sizes the matrix-core kernel takes runs it for both kinds of attention (and the model of
+    odd sizes runs the generic one where they do not fit)."""
+    from kestrel_amd.ops import fast
+
+    calls = []
+    original = fast.attention_biased_bf16
+
+    def spy(*args, **kwargs):
+        done = original(*args, **kwargs)
+        calls.append((kwargs.get("maps", 1), bool(kwargs.get("values_in_keys")), done))
+        return done
+
+    fast.attention_biased_bf16 = spy
+    try:
+        for name, expect in (("P", True), ("Q", False)):
+            calls.clear()
+            folder = cases.model_dir(name)
+            runner = _runner(folder, torch.bfloat16)
+            reqs = {"r": Request("r", _ids(folder, 900, 40))}
+            helpers.replay(runner, reqs, [[("r", 39)], [("r", 1)]])
+            assert {(m, v) for m, v, _ in calls} == {(2, False), (1, True)}
+            if expect:              # (its second latent layer's rows are wider than the kernel takes)
+                assert (2, False, True) in calls and (1, True, True) in calls, calls
+            else:                   # (maps of 20 and 28 channels; its first latent layer's rows of 48 the kernel takes)
+                assert not any(done for m, _, done in calls if m == 2) and (1, True, False) in calls, calls
+    finally:
+        fast.attention_biased_bf16 = original
