@@ -130,8 +130,13 @@ __device__ __forceinline__ float sp_conv_at(const ConvArgs& a, int t, int local,
     return acc;
 }
 
+constexpr int SP_MAX_ROT = 1024;
+
+// A workgroup per token. The angles of a token are the same for every head: their cosines and sines are computed once,
+// into LDS. Of a rotated pair of channels the thread of the first computes both convolutions and writes both results.
 template <typename T>
 __global__ void __launch_bounds__(SP_THREADS) conv_prepare_kernel(ConvArgs a) {
+    __shared__ float cs[SP_MAX_ROT / 2], sn[SP_MAX_ROT / 2];
     const int t = blockIdx.x;
     const int r = a.token_row[t];
     const int local = t - a.cu_q[r];
@@ -140,30 +145,36 @@ __global__ void __launch_bounds__(SP_THREADS) conv_prepare_kernel(ConvArgs a) {
     const float place = (float)a.positions[t];
     const int at = a.slots ? a.slots[t] : -1;
     const int page = at >= 0 ? at / a.page_size : 0, off = at >= 0 ? at % a.page_size : 0;
+    const int half = a.rot / 2;
+    if (a.freqs) {
+        for (int i = threadIdx.x; i < half; i += SP_THREADS) sincosf(place * a.freqs[i], &sn[i], &cs[i]);
+        __syncthreads();
+    }
+    T* q_out = reinterpret_cast<T*>(a.q_out) + (size_t)t * a.q_stride;
+    T* k_out = reinterpret_cast<T*>(a.k_cache) + ((size_t)page * a.Hk * a.page_size + off) * a.hd;
     for (int c = threadIdx.x; c < a.C; c += SP_THREADS) {
-        float y = sp_conv_at<T>(a, t, local, slot, c);
         if (c < Cq + Ck) {
             const int within = c < Cq ? c : c - Cq;
             const int head = within / a.hd, d = within % a.hd;
+            T* dst = c < Cq ? q_out + c : (at >= 0 ? k_out + (size_t)head * a.page_size * a.hd + d : nullptr);
             if (a.freqs && d < a.rot) {
-                const int half = a.rot / 2;
                 const bool first = a.interleaved ? (d & 1) == 0 : d < half;
-                const int partner = a.interleaved ? (d ^ 1) : (first ? d + half : d - half);
-                const int i = a.interleaved ? d / 2 : (first ? d : d - half);
-                const float other = sp_conv_at<T>(a, t, local, slot, c - d + partner);
-                const float angle = place * a.freqs[i];
-                const float cs = cosf(angle), sn = sinf(angle);
-                y = first ? y * cs - other * sn : y * cs + other * sn;
-            }
-            if (c < Cq) {
-                reinterpret_cast<T*>(a.q_out)[(size_t)t * a.q_stride + c] = ka_from_float<T>(y);
-            } else if (at >= 0) {
-                reinterpret_cast<T*>(a.k_cache)[(((size_t)page * a.Hk + head) * a.page_size + off) * a.hd + d] = ka_from_float<T>(y);
+                if (!first) continue;                   // (written by the thread of its partner)
+                const int step = a.interleaved ? 1 : half;
+                const int i = a.interleaved ? d / 2 : d;
+                const float y = sp_conv_at<T>(a, t, local, slot, c), other = sp_conv_at<T>(a, t, local, slot, c + step);
+                if (dst) {
+                    dst[0] = ka_from_float<T>(y * cs[i] - other * sn[i]);
+                    dst[step] = ka_from_float<T>(other * cs[i] + y * sn[i]);
+                }
+            } else if (dst) {
+                *dst = ka_from_float<T>(sp_conv_at<T>(a, t, local, slot, c));
             }
         } else if (at >= 0) {
             const int within = c - Cq - Ck;
             const int head = within / a.hdv, d = within % a.hdv;
-            reinterpret_cast<T*>(a.v_cache)[(((size_t)page * a.Hv + head) * a.hdv + d) * a.page_size + off] = ka_from_float<T>(y);
+            reinterpret_cast<T*>(a.v_cache)[(((size_t)page * a.Hv + head) * a.hdv + d) * a.page_size + off] =
+                ka_from_float<T>(sp_conv_at<T>(a, t, local, slot, c));
         }
     }
 }
@@ -195,7 +206,7 @@ KA_API int ka_conv_prepare(const void* u, int dtype, long u_stride, const float*
     KA_CHECK(dtype == KA_F32 || dtype == KA_BF16, "ka_conv_prepare: unsupported dtype %d", dtype);
     KA_CHECK(K == 0 || taps != nullptr, "ka_conv_prepare: taps missing");
     KA_CHECK(K <= 1 || state != nullptr, "ka_conv_prepare: a convolution of %d taps needs its state", K);
-    KA_CHECK(freqs == nullptr || (rot > 0 && rot % 2 == 0 && rot <= hd), "ka_conv_prepare: rotation of %d channels of %d", rot, hd);
+    KA_CHECK(freqs == nullptr || (rot > 0 && rot % 2 == 0 && rot <= hd && rot <= SP_MAX_ROT), "ka_conv_prepare: rotation of %d channels of %d", rot, hd);
     KA_CHECK(slots == nullptr || (k_cache != nullptr && v_cache != nullptr), "ka_conv_prepare: cache tensors missing");
     ConvArgs a;
     a.u = u; a.u_stride = u_stride; a.taps = taps; a.state = state; a.K = K;

@@ -59,6 +59,8 @@ _SIGNATURES = {
                                  _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_long, _c_float,
                                  _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_void_p, _c_int, _c_void_p, _c_long,
                                  _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_void_p],
+    "ka_heads_linear_bf16": [_c_void_p, _c_long, _c_int, _c_void_p, _c_void_p, _c_long, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void_p],
+    "ka_heads_linear_supported": [_c_long, _c_int, _c_long, _c_int, _c_int, _c_int],
     "ka_matrix_memory_chunks_bf16": [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_long, _c_void_p, _c_void_p, _c_void_p, _c_void_p,
                                      _c_void_p, _c_void_p, _c_long, _c_int, _c_int, _c_int, _c_int, _c_float, _c_float, _c_float,
                                      _c_void_p, _c_int, _c_void_p],
@@ -692,6 +694,28 @@ def attention_latent_bf16(q, cache, block_table, token_row, kv_hi, out, scale, n
     value, with a sink score per head, on the matrix cores. False: not covered (rows above 128 channels among others)."""
     return attention_biased_bf16(q, cache, None, block_table, token_row, None, kv_hi, out, scale, n_heads, 1, row_dim, rank,
                                  None, None, None, batch, sinks=sinks, values_in_keys=True)
+
+
+def heads_linear_bf16(a, a_head: int, k: int, weights, out, out_head: int, n_out: int) -> bool:
+    """``out[:, h, :n_out] = a[:, h, :k] @ weights[h].T`` for every head in one launch on the matrix cores: ``a`` ``[n, H a_head]``,
+    ``weights`` ``[H, n_out, k]``, ``out`` ``[n, H out_head]``, all bf16. False: not covered (``k`` no multiple of 16, heads
+    that are not aligned), nothing was run."""
+    n = a.shape[0]
+    if n == 0:
+        return True
+    heads = int(weights.shape[0])
+    if a.dtype != torch.bfloat16 or out.dtype != torch.bfloat16 or weights.dtype != torch.bfloat16 or a.stride(1) != 1 \
+            or out.stride(1) != 1 or not weights.is_contiguous() or tuple(weights.shape) != (heads, n_out, k) \
+            or a.shape[1] < heads * a_head or out.shape[1] < heads * out_head or n > 64 * 65535:
+        return False
+    lda, ldo = (a.stride(0), out.stride(0)) if n > 1 else (heads * a_head, heads * out_head)
+    handle = lib()
+    if a.data_ptr() % 16 or out.data_ptr() % 8 or weights.data_ptr() % 16 \
+            or not handle.ka_heads_linear_supported(lda, a_head, ldo, out_head, n_out, k):
+        return False
+    _check(handle.ka_heads_linear_bf16(a.data_ptr(), lda, a_head, weights.data_ptr(), out.data_ptr(), ldo, out_head, n, heads,
+                                       n_out, k, stream_ptr()))
+    return True
 
 
 def matrix_memory_chunks_scratch(n: int, n_rows: int, n_heads: int, head_dim: int, value_dim: int) -> int:

@@ -101,8 +101,38 @@ def _parallel(block: "Block", x, batch, cache, normed=None, then=None):
 _parallel.hands_over = True
 
 
+def _sequential_few_rows(block: "Block", x, batch, cache) -> bool:
+    """The sequential block for a few bf16 rows: each norm in the prologue of the launch that reads it (the mixer's first
+    linear; the feed-forward's first linear where it offers ``from_stream``). Needs a root-mean-square norm and a mixer
+    that offers its stages; returns ``False`` (nothing was run) otherwise."""
+    from ..ops import fast
+    from ..ops.linear import linear
+
+    n = x.shape[0]
+    if block.dtype != torch.bfloat16 or n > fast.SKINNY_LN_MAX_ROWS or not fast.FUSE_LAYERNORM_PROLOGUE:
+        return False
+    rms = block.norm.rms_operands() if callable(getattr(block.norm, "rms_operands", None)) else None
+    m_in, m_out = block.mixer.input_projection(), block.mixer.output_projection()
+    if rms is None or m_in is None or m_out is None:
+        return False
+    ws = batch.workspace
+    projected = ws.get("block.mixer_in", (n, m_in[2]), block.dtype)
+    if not fast.layernorm_linear(x, rms[0], None, rms[1], m_in[0], m_in[1], projected, 0, centred=False):
+        return False
+    linear(block.mixer.attend(projected, batch, cache), m_out[0], m_out[1], x, accumulate=True)
+    if block.feed_forward is not None:
+        from_stream = getattr(block.feed_forward, "from_stream", None)
+        if from_stream is None or not from_stream(x, block.norm2, batch):
+            h = ws.get("block.h", tuple(x.shape), block.dtype)
+            block.norm2.forward(x, h)
+            block.feed_forward.forward(h, batch, x)
+    return True
+
+
 def _sequential(block: "Block", x, batch, cache) -> None:
     """``x += mixer(norm(x)); x += ff(norm2(x))``; without a feed-forward the first half only."""
+    if _sequential_few_rows(block, x, batch, cache):
+        return
     h = batch.workspace.get("block.h", tuple(x.shape), block.dtype)
     block.norm.forward(x, h)
     block.mixer.forward(h, batch, cache, x)

@@ -100,7 +100,10 @@ class DifferentialAttention(Mixer):
         return fast.biased_query_block(self.spec.head_dim, self.spec.value_dim)
 
     def input_projection(self):
-        return None        # (the block runs this mixer through ``forward``)
+        return self.in_weight, None, self.in_dim
+
+    def output_projection(self):
+        return self.proj_weight, None
 
     def attend(self, projected, batch, cache: LayerCache, beside=None) -> torch.Tensor:
         """Convolution, rotation, cache write, both maps, their combination; returns the input of the output projection."""

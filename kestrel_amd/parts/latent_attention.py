@@ -91,6 +91,12 @@ class LatentAttention(Mixer):
         from ..ops import fast
         return fast.biased_query_block(self.row_dim, self.spec.kv_rank)
 
+    def input_projection(self):
+        return self.down_weight, None, self.down_dim
+
+    def output_projection(self):
+        return self.proj_weight, None
+
     def attend(self, down, batch, cache: LayerCache, beside=None) -> torch.Tensor:
         """From the projected row ``[c_q' | c' | k_r | gate]`` to the gated heads, the input of the output projection."""
         spec = self.spec

@@ -126,6 +126,23 @@ class ClampedGatedFeedForward(GatedFeedForward):
     def output_projection(self):
         return None
 
+    def from_stream(self, x, norm, batch) -> bool:
+        """The feed-forward of ``norm(x)`` added into fp32 ``x`` with the norm in the prologue of the first linear's launch
+        (a few bf16 rows, a root-mean-square norm); ``False``: not covered, nothing was run."""
+        from ..ops import core, fast
+        spec = self.spec
+        rms = norm.rms_operands() if callable(getattr(norm, "rms_operands", None)) else None
+        if rms is None or self.dtype != torch.bfloat16:
+            return False
+        n = x.shape[0]
+        sums = batch.workspace.get("ff.pair_sums", (n, 2 * spec.hidden_dim), self.dtype)
+        if not fast.layernorm_linear(x, rms[0], None, rms[1], self.pairs, self.pair_bias, sums, 0, centred=False):
+            return False
+        hidden = batch.workspace.get("ff.hidden", (n, spec.hidden_dim), self.dtype)
+        core.clamped_pairs(sums, hidden, spec.limit, spec.slope, spec.shift)
+        linear(hidden, self.down_weight, self.down_bias, x, accumulate=True)
+        return True
+
     def forward(self, h, batch, residual) -> None:
         from ..ops import core
         spec = self.spec

@@ -766,3 +766,23 @@ def test_the_matrix_core_kernels_run_where_sizes_allow():
                 assert not any(done for m, _, done in calls if m == 2) and (1, True, False) in calls, calls
     finally:
         fast.attention_biased_bf16 = original
+
+
+@pytest.mark.parametrize("n", [1, 8, 70, 300])
+@pytest.mark.parametrize("heads, a_head, k, out_head, n_out", [(5, 72, 64, 112, 96), (3, 32, 32, 40, 40), (16, 96, 96, 64, 64),
+                                                                 (2, 144, 128, 20, 20), (7, 16, 16, 8, 6)])
+def test_a_linear_per_head_on_the_matrix_cores(heads, a_head, k, out_head, n_out, n):
+    """Every head's own matrix in one launch: heads that read the first ``k`` channels of their part of a row and write the
+    first ``n_out`` of theirs; what lies behind is left as it was."""
+    from kestrel_amd.ops import fast
+
+    g = _gen(8)
+    bf = torch.bfloat16
+    a = torch.randn(n, heads * a_head + 8, generator=g).to(bf)
+    w = (torch.randn(heads, n_out, k, generator=g) / math.sqrt(k)).to(bf)
+    out = torch.full((n, heads * out_head), 7.0, dtype=bf, device=DEV)
+    assert fast.heads_linear_bf16(a.to(DEV)[:, :heads * a_head], a_head, k, w.to(DEV), out, out_head, n_out)
+    got = out.double().cpu().view(n, heads, out_head)
+    want = torch.einsum("nhk,hok->nho", a[:, :heads * a_head].double().view(n, heads, a_head)[:, :, :k], w.double())
+    assert torch.allclose(got[:, :, :n_out], want, rtol=2e-2, atol=2e-2)
+    assert bool((got[:, :, n_out:] == 7.0).all())
