@@ -1,6 +1,7 @@
 // A linear per head on the matrix cores: out[r, h, o] = sum_k a[r, h, k] * w[h, o, k] for every head h, with rows of `a`
 // that hold heads of `a_head` channels (the first k of each are read) and rows of `out` that hold heads of `out_head`
-// channels (the first n_out of each are written, the rest are left alone). bf16 in and out, sums in fp32.
+// channels (the first n_out of each are written, the rest are left alone). bf16 in and out, sums in fp32. With `gate`
+// (rows laid out as those of `out`, a row stride of their own) every output is multiplied by the sigmoid of its gate.
 //
 // What it is for: mixers that keep a low-rank latent per key and move the per-head up-projections to the query's side
 // (every head's query times its own key matrix, every head's weighted sum of latents times its own value matrix). One
@@ -20,7 +21,7 @@ constexpr int HL_TILE = 64;
 
 __global__ void __launch_bounds__(256)
 heads_linear_kernel(const bf16_t* __restrict__ a, long lda, int a_head, const bf16_t* __restrict__ w, bf16_t* __restrict__ out,
-                    long ldo, int out_head, int n, int n_out, int k) {
+                    long ldo, int out_head, int n, int n_out, int k, const bf16_t* __restrict__ gate, long ldg) {
     const int wave = threadIdx.x / KA_WAVE, lane = threadIdx.x % KA_WAVE;
     const int col = lane % 32, half = lane / 32;
     const int head = blockIdx.z;
@@ -40,6 +41,14 @@ heads_linear_kernel(const bf16_t* __restrict__ a, long lda, int a_head, const bf
     if (row >= n) return;
     // register i: output o0 + (i / 4) * 8 + half * 4 + i % 4 of the lane's row
     bf16_t* op = out + (size_t)row * ldo + (size_t)head * out_head;
+    if (gate) {
+        const bf16_t* gp = gate + (size_t)row * ldg + (size_t)head * out_head;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            const int o = o0 + (i / 4) * 8 + half * 4 + i % 4;
+            if (o < n_out) acc[i] *= 1.0f / (1.0f + __expf(-(float)gp[o]));
+        }
+    }
 #pragma unroll
     for (int g4 = 0; g4 < 4; ++g4) {
         const int o = o0 + g4 * 8 + half * 4;
@@ -63,7 +72,7 @@ KA_API int ka_heads_linear_supported(long lda, int a_head, long ldo, int out_hea
 }
 
 KA_API int ka_heads_linear_bf16(const void* a, long lda, int a_head, const void* w, void* out, long ldo, int out_head, int n,
-                                int heads, int n_out, int k, hipStream_t stream) {
+                                int heads, int n_out, int k, const void* gate, long ldg, hipStream_t stream) {
     const char* who = "ka_heads_linear_bf16";
     KA_CHECK(n >= 0 && heads > 0 && heads <= 65535, "%s: bad sizes", who);
     KA_CHECK(ka_heads_linear_supported(lda, a_head, ldo, out_head, n_out, k), "%s: sizes k=%d n_out=%d heads of %d -> %d not covered", who, k, n_out, a_head, out_head);
@@ -73,7 +82,7 @@ KA_API int ka_heads_linear_bf16(const void* a, long lda, int a_head, const void*
     const dim3 grid((n_out + HL_TILE - 1) / HL_TILE, (n + HL_TILE - 1) / HL_TILE, heads);
     KA_CHECK(grid.y <= 65535, "%s: too many rows %d", who, n);
     hipLaunchKernelGGL(heads_linear_kernel, grid, dim3(256), 0, stream, (const bf16_t*)a, lda, a_head, (const bf16_t*)w,
-                       (bf16_t*)out, ldo, out_head, n, n_out, k);
+                       (bf16_t*)out, ldo, out_head, n, n_out, k, (const bf16_t*)gate, ldg);
     KA_LAUNCH_CHECK();
     return 0;
 }

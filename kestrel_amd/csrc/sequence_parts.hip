@@ -132,8 +132,9 @@ __device__ __forceinline__ float sp_conv_at(const ConvArgs& a, int t, int local,
 
 constexpr int SP_MAX_ROT = 1024;
 
-// A workgroup per token. The angles of a token are the same for every head: their cosines and sines are computed once,
-// into LDS. Of a rotated pair of channels the thread of the first computes both convolutions and writes both results.
+// Grid (tokens, blocks of SP_THREADS channels): a thread per token and channel. The angles of a token are the same for
+// every head: a workgroup computes their cosines and sines once, into LDS. Of a rotated pair of channels the thread of the
+// first computes both convolutions and writes both results.
 template <typename T>
 __global__ void __launch_bounds__(SP_THREADS) conv_prepare_kernel(ConvArgs a) {
     __shared__ float cs[SP_MAX_ROT / 2], sn[SP_MAX_ROT / 2];
@@ -152,14 +153,16 @@ __global__ void __launch_bounds__(SP_THREADS) conv_prepare_kernel(ConvArgs a) {
     }
     T* q_out = reinterpret_cast<T*>(a.q_out) + (size_t)t * a.q_stride;
     T* k_out = reinterpret_cast<T*>(a.k_cache) + ((size_t)page * a.Hk * a.page_size + off) * a.hd;
-    for (int c = threadIdx.x; c < a.C; c += SP_THREADS) {
+    {
+        const int c = blockIdx.y * SP_THREADS + threadIdx.x;
+        if (c >= a.C) return;
         if (c < Cq + Ck) {
             const int within = c < Cq ? c : c - Cq;
             const int head = within / a.hd, d = within % a.hd;
             T* dst = c < Cq ? q_out + c : (at >= 0 ? k_out + (size_t)head * a.page_size * a.hd + d : nullptr);
             if (a.freqs && d < a.rot) {
                 const bool first = a.interleaved ? (d & 1) == 0 : d < half;
-                if (!first) continue;                   // (written by the thread of its partner)
+                if (!first) return;                     // (written by the thread of its partner)
                 const int step = a.interleaved ? 1 : half;
                 const int i = a.interleaved ? d / 2 : d;
                 const float y = sp_conv_at<T>(a, t, local, slot, c), other = sp_conv_at<T>(a, t, local, slot, c + step);
@@ -188,7 +191,9 @@ __global__ void __launch_bounds__(SP_THREADS) conv_state_kernel(ConvArgs a) {
     const T* u = reinterpret_cast<const T*>(a.u);
     const int keep = a.K - 1;
     float* st = a.state + (size_t)slot * keep * a.C;
-    for (int c = threadIdx.x; c < a.C; c += SP_THREADS) {
+    {
+        const int c = blockIdx.y * SP_THREADS + threadIdx.x;
+        if (c >= a.C) return;
         // entry s stands for the place s - keep relative to the next step's first token; in rising order an entry is
         // read (s + q) before it is written
         for (int s = 0; s < keep; ++s) {
@@ -217,12 +222,14 @@ KA_API int ka_conv_prepare(const void* u, int dtype, long u_stride, const float*
     a.Hq = Hq; a.Hk = Hk; a.hd = hd; a.Hv = Hv; a.hdv = hdv; a.page_size = page_size;
     a.freqs = freqs; a.rot = freqs ? rot : 0; a.interleaved = interleaved;
     if (n == 0) return 0;
-    if (dtype == KA_F32) hipLaunchKernelGGL(conv_prepare_kernel<float>, dim3(n), dim3(SP_THREADS), 0, stream, a);
-    else hipLaunchKernelGGL(conv_prepare_kernel<bf16_t>, dim3(n), dim3(SP_THREADS), 0, stream, a);
+    const int blocks = (a.C + SP_THREADS - 1) / SP_THREADS;
+    KA_CHECK(blocks <= 65535, "ka_conv_prepare: too many channels %d", a.C);
+    if (dtype == KA_F32) hipLaunchKernelGGL(conv_prepare_kernel<float>, dim3(n, blocks), dim3(SP_THREADS), 0, stream, a);
+    else hipLaunchKernelGGL(conv_prepare_kernel<bf16_t>, dim3(n, blocks), dim3(SP_THREADS), 0, stream, a);
     KA_LAUNCH_CHECK();
     if (K > 1 && n_rows > 0) {
-        if (dtype == KA_F32) hipLaunchKernelGGL(conv_state_kernel<float>, dim3(n_rows), dim3(SP_THREADS), 0, stream, a);
-        else hipLaunchKernelGGL(conv_state_kernel<bf16_t>, dim3(n_rows), dim3(SP_THREADS), 0, stream, a);
+        if (dtype == KA_F32) hipLaunchKernelGGL(conv_state_kernel<float>, dim3(n_rows, blocks), dim3(SP_THREADS), 0, stream, a);
+        else hipLaunchKernelGGL(conv_state_kernel<bf16_t>, dim3(n_rows, blocks), dim3(SP_THREADS), 0, stream, a);
         KA_LAUNCH_CHECK();
     }
     return 0;

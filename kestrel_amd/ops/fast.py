@@ -59,7 +59,8 @@ _SIGNATURES = {
                                  _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_long, _c_float,
                                  _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_void_p, _c_int, _c_void_p, _c_long,
                                  _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_void_p],
-    "ka_heads_linear_bf16": [_c_void_p, _c_long, _c_int, _c_void_p, _c_void_p, _c_long, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void_p],
+    "ka_heads_linear_bf16": [_c_void_p, _c_long, _c_int, _c_void_p, _c_void_p, _c_long, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void_p,
+                             _c_long, _c_void_p],
     "ka_heads_linear_supported": [_c_long, _c_int, _c_long, _c_int, _c_int, _c_int],
     "ka_matrix_memory_chunks_bf16": [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_long, _c_void_p, _c_void_p, _c_void_p, _c_void_p,
                                      _c_void_p, _c_void_p, _c_long, _c_int, _c_int, _c_int, _c_int, _c_float, _c_float, _c_float,
@@ -696,10 +697,10 @@ def attention_latent_bf16(q, cache, block_table, token_row, kv_hi, out, scale, n
                                  None, None, None, batch, sinks=sinks, values_in_keys=True)
 
 
-def heads_linear_bf16(a, a_head: int, k: int, weights, out, out_head: int, n_out: int) -> bool:
+def heads_linear_bf16(a, a_head: int, k: int, weights, out, out_head: int, n_out: int, gate=None) -> bool:
     """``out[:, h, :n_out] = a[:, h, :k] @ weights[h].T`` for every head in one launch on the matrix cores: ``a`` ``[n, H a_head]``,
-    ``weights`` ``[H, n_out, k]``, ``out`` ``[n, H out_head]``, all bf16. False: not covered (``k`` no multiple of 16, heads
-    that are not aligned), nothing was run."""
+    ``weights`` ``[H, n_out, k]``, ``out`` ``[n, H out_head]``, all bf16; with ``gate`` (bf16, laid out as ``out``) times the
+    sigmoid of it. False: not covered (``k`` no multiple of 16, heads that are not aligned), nothing was run."""
     n = a.shape[0]
     if n == 0:
         return True
@@ -709,12 +710,16 @@ def heads_linear_bf16(a, a_head: int, k: int, weights, out, out_head: int, n_out
             or a.shape[1] < heads * a_head or out.shape[1] < heads * out_head or n > 64 * 65535:
         return False
     lda, ldo = (a.stride(0), out.stride(0)) if n > 1 else (heads * a_head, heads * out_head)
+    if gate is not None and (gate.dtype != torch.bfloat16 or gate.dim() != 2 or gate.stride(1) != 1 or gate.shape[0] != n
+                             or gate.shape[1] < heads * out_head):
+        return False
     handle = lib()
     if a.data_ptr() % 16 or out.data_ptr() % 8 or weights.data_ptr() % 16 \
             or not handle.ka_heads_linear_supported(lda, a_head, ldo, out_head, n_out, k):
         return False
     _check(handle.ka_heads_linear_bf16(a.data_ptr(), lda, a_head, weights.data_ptr(), out.data_ptr(), ldo, out_head, n, heads,
-                                       n_out, k, stream_ptr()))
+                                       n_out, k, _ptr(gate), (gate.stride(0) if n > 1 else heads * out_head) if gate is not None else 0,
+                                       stream_ptr()))
     return True
 
 

@@ -122,10 +122,9 @@ class DifferentialAttention(Mixer):
         done = False
         if self.dtype == torch.bfloat16:
             from ..ops import fast
-            mapped = getattr(fast, "attention_maps_bf16", None)
-            if mapped is not None:
-                done = mapped(q, cache.k, cache.v, group.block_table, batch.token_row, group.kv_lo, batch.kv_hi, maps, float(spec.scale),
-                              2 * spec.n_heads, 2 * spec.n_kv_heads, spec.head_dim, spec.value_dim, self.keep_first, 2, batch)
+            done = fast.attention_maps_bf16(q, cache.k, cache.v, group.block_table, batch.token_row, group.kv_lo, batch.kv_hi, maps,
+                                            float(spec.scale), 2 * spec.n_heads, 2 * spec.n_kv_heads, spec.head_dim, spec.value_dim,
+                                            self.keep_first, 2, batch)
         if not done:
             core.attention_generic(q, cache.k, cache.v, group.block_table, batch.token_row, group.kv_lo, batch.kv_hi, maps,
                                    float(spec.scale), 2 * spec.n_heads, 2 * spec.n_kv_heads, spec.head_dim, spec.value_dim,

@@ -117,30 +117,28 @@ class LatentAttention(Mixer):
         done = False
         if self.dtype == torch.bfloat16:
             from ..ops import fast
-            latent = getattr(fast, "attention_latent_bf16", None)
-            if latent is not None:
-                done = latent(full, cache.k, group.block_table, batch.token_row, batch.kv_hi, mixed, float(spec.scale), spec.n_heads,
-                              self.row_dim, spec.kv_rank, self._sinks, batch)
+            done = fast.attention_latent_bf16(full, cache.k, group.block_table, batch.token_row, batch.kv_hi, mixed, float(spec.scale),
+                                              spec.n_heads, self.row_dim, spec.kv_rank, self._sinks, batch)
         if not done:
             core.attention_generic(full, cache.k, None, group.block_table, batch.token_row, group.kv_lo, batch.kv_hi, mixed,
                                    float(spec.scale), spec.n_heads, 1, self.row_dim, spec.kv_rank, sinks=self._sinks,
                                    values_in_keys=True)
         heads = ws.get("latent.heads", (n, self.out_dim), self.dtype)
-        self._per_head(mixed, spec.kv_rank, spec.kv_rank, self.lift, heads, spec.value_dim, spec.value_dim)
-        if gate is not None:
+        if not self._per_head(mixed, spec.kv_rank, spec.kv_rank, self.lift, heads, spec.value_dim, spec.value_dim, gate) \
+                and gate is not None:
             core.gate_mul(heads, gate)
         return heads
 
-    def _per_head(self, a, a_head: int, k: int, weights, out, out_head: int, n_out: int) -> None:
+    def _per_head(self, a, a_head: int, k: int, weights, out, out_head: int, n_out: int, gate=None) -> bool:
         """``out[:, h, :n_out] = a[:, h, :k] @ weights[h].T`` for every head (rows of ``a`` hold heads of ``a_head`` channels, rows of
-        ``out`` heads of ``out_head``)."""
+        ``out`` heads of ``out_head``). True: the outputs were also multiplied by the sigmoid of ``gate``."""
         if self.dtype == torch.bfloat16:
             from ..ops import fast
-            batched = getattr(fast, "heads_linear_bf16", None)
-            if batched is not None and batched(a, a_head, k, weights, out, out_head, n_out):
-                return
+            if fast.heads_linear_bf16(a, a_head, k, weights, out, out_head, n_out, gate):
+                return gate is not None
         for h in range(self.spec.n_heads):
             linear(a[:, h * a_head:h * a_head + k], weights[h], None, out[:, h * out_head:h * out_head + n_out])
+        return False
 
     def mix(self, h, batch, cache: LayerCache, out, accumulate: bool) -> None:
         down = batch.workspace.get("latent.down", (h.shape[0], self.down_dim), self.dtype)

@@ -786,3 +786,9 @@ def test_a_linear_per_head_on_the_matrix_cores(heads, a_head, k, out_head, n_out
     want = torch.einsum("nhk,hok->nho", a[:, :heads * a_head].double().view(n, heads, a_head)[:, :, :k], w.double())
     assert torch.allclose(got[:, :, :n_out], want, rtol=2e-2, atol=2e-2)
     assert bool((got[:, :, n_out:] == 7.0).all())
+    # with a gate in a buffer of wider rows: times its sigmoid
+    gate = (torch.randn(n, heads * out_head + 24, generator=g) * 2).to(bf)
+    assert fast.heads_linear_bf16(a.to(DEV)[:, :heads * a_head], a_head, k, w.to(DEV), out, out_head, n_out, gate.to(DEV)[:, 24:])
+    got = out.double().cpu().view(n, heads, out_head)
+    want = want * torch.sigmoid(gate[:, 24:].double().view(n, heads, out_head)[:, :, :n_out])
+    assert torch.allclose(got[:, :, :n_out], want, rtol=2e-2, atol=2e-2)
