@@ -24,6 +24,12 @@
 //    and values at once); the value operand is then gathered from the key page;
 //  * out_f32: outputs leave as fp32.
 //
+// Heads wider than 128 channels (latent rows of several hundred numbers) take the same loop in its wide form (NK = 0):
+// the head size is a run-time number, the queries of the workgroup's 32 columns lie in LDS instead of registers (every
+// wave reads them from there, 16 bytes a lane and step), keys are streamed step by step, and a workgroup owns a slice of
+// 128 value channels (blockIdx.z counts the slices; every slice computes the scores again, which costs little where
+// the keys are what is waited for).
+//
 // A workgroup owns 32 columns of the score product and one kv head. In a step with prompt portions a
 // column is a query of a block of 32 consecutive tokens of one row and one query head (the host lists the
 // blocks); in a decode step, where every row has one token, the columns are the query heads that share the
@@ -58,7 +64,8 @@ __device__ __forceinline__ float ab_sum_halves(float x) {
     return __uint_as_float(r[0]) + __uint_as_float(r[1]);
 }
 
-// NK: 16-channel steps of a query/key head (hd = 16 NK); NV: 32-channel blocks of a value head (hdv <= 32 NV).
+// NK: 16-channel steps of a query/key head (hd = 16 NK; NK = 0: hd_wide channels, see above); NV: 32-channel blocks of a
+// value head (hdv <= 32 NV, or, in the wide form, the slice of the value head that blockIdx.z names).
 // heads_per_block: 1 = the columns are consecutive tokens of a block of queries (qblk_row / qblk_tok list the blocks,
 // grid (H, blocks)); > 1 = a decode step, the columns are that many query heads of one kv head of token blockIdx.y
 // (grid (Hkv * ceil(G / heads_per_block), tokens)).
@@ -72,8 +79,10 @@ attn_biased_kernel(const bf16_t* __restrict__ q, long q_row_stride, const bf16_t
                    long out_row_stride, float scale, int H, int Hkv, int hdv, int heads_per_block, int has_sink,
                    float sink_score, const float* __restrict__ bias_table, int bias_len, const bf16_t* __restrict__ gate,
                    long gate_row_stride, const float* __restrict__ sinks, int keep_first, int maps, int values_in_keys,
-                   int out_f32) {
-    constexpr int HD = NK * 16;
+                   int out_f32, int hd_wide) {
+    constexpr bool WIDE = NK == 0;
+    const int HD = WIDE ? hd_wide : NK * 16;
+    const int v0 = WIDE ? blockIdx.z * (NV * 32) : 0;     // the first value channel of this workgroup's slice
     constexpr int REC = 16 * NV + 2;            // floats a lane hands over at a merge: its outputs, m and l
     extern __shared__ float mrg[];              // [waves / 2][REC][64]
     const int n_waves = blockDim.x / KA_WAVE;
@@ -115,11 +124,17 @@ attn_biased_kernel(const bf16_t* __restrict__ q, long q_row_stride, const bf16_t
     max_lo = __builtin_amdgcn_readfirstlane(max_lo);
 
     // queries: the column operand of the score product, held for the whole loop
-    ab_bf16x8 qreg[NK];
+    ab_bf16x8 qreg[WIDE ? 1 : NK];
+    ab_bf16x8* q_lds = reinterpret_cast<ab_bf16x8*>(mrg + (size_t)(n_waves / 2) * REC * KA_WAVE);     // [hd / 16][64]
     {
         const bf16_t* qp = q + (size_t)tok * q_row_stride + (size_t)head * HD + half * 8;
+        if constexpr (WIDE) {
+            for (int c = wave; c < HD / 16; c += n_waves) q_lds[c * KA_WAVE + lane] = *reinterpret_cast<const ab_bf16x8*>(qp + c * 16);
+            __syncthreads();
+        } else {
 #pragma unroll
-        for (int c = 0; c < NK; ++c) qreg[c] = *reinterpret_cast<const ab_bf16x8*>(qp + c * 16);
+            for (int c = 0; c < NK; ++c) qreg[c] = *reinterpret_cast<const ab_bf16x8*>(qp + c * 16);
+        }
     }
     const float slope2 = slopes ? slopes[head] * AB_LOG2E : 0.f;     // in powers of two, like everything below
     const float scale2 = scale * AB_LOG2E;
@@ -146,7 +161,7 @@ attn_biased_kernel(const bf16_t* __restrict__ q, long q_row_stride, const bf16_t
     // the value rows (channels) this lane loads: clamped into the head where the last block is not full
     int vch[NV];
 #pragma unroll
-    for (int b = 0; b < NV; ++b) vch[b] = min(b * 32 + col, hdv - 1);
+    for (int b = 0; b < NV; ++b) vch[b] = min(v0 + b * 32 + col, hdv - 1);
 
     if (blk_lo < blk_hi) {
         const int first_tile = blk_lo / AB_TILE, last_tile = (blk_hi - 1) / AB_TILE;
@@ -163,9 +178,9 @@ attn_biased_kernel(const bf16_t* __restrict__ q, long q_row_stride, const bf16_t
                 const int e = table[min(tile * 2 + p, max_pages - 1)];
                 pg[p] = e < 0 ? 0 : e;
             }
-            ab_bf16x8 kr[NK];
-            {
-                const bf16_t* kp = k_cache + (size_t)pg[kpage_in_tile] * k_page + k_head + (size_t)kslot * HD + half * 8;
+            ab_bf16x8 kr[WIDE ? 1 : NK];
+            const bf16_t* kp = k_cache + (size_t)pg[kpage_in_tile] * k_page + k_head + (size_t)kslot * HD + half * 8;
+            if constexpr (!WIDE) {
 #pragma unroll
                 for (int c = 0; c < NK; ++c) kr[c] = *reinterpret_cast<const ab_bf16x8*>(kp + c * 16);
             }
@@ -191,8 +206,15 @@ attn_biased_kernel(const bf16_t* __restrict__ q, long q_row_stride, const bf16_t
             ab_floatx16 s;
 #pragma unroll
             for (int i = 0; i < 16; ++i) s[i] = 0.f;
+            if constexpr (WIDE) {
+
+                for (int c = 0; c < HD / 16; ++c)
+                    s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(*reinterpret_cast<const ab_bf16x8*>(kp + c * 16),
+                                                                q_lds[c * KA_WAVE + lane], s, 0, 0, 0);
+            } else {
 #pragma unroll
-            for (int c = 0; c < NK; ++c) s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kr[c], qreg[c], s, 0, 0, 0);
+                for (int c = 0; c < NK; ++c) s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kr[c], qreg[c], s, 0, 0, 0);
+            }
             // register i of this lane: key base + (i / 8) * 16 + half * 8 + i % 8 of the lane's column
             const int j0 = base + half * 8;
             const float bias0 = -slope2 * (float)(place - j0);          // (an integer distance: exact)
@@ -296,7 +318,7 @@ attn_biased_kernel(const bf16_t* __restrict__ q, long q_row_stride, const bf16_t
             for (int i = 0; i < 16; ++i) o[b][i] *= c;
     }
     const float inv = l > 0.f ? 1.0f / l : 0.f;
-    // register i of block b: channel b * 32 + (i / 4) * 8 + half * 4 + i % 4 of the lane's column
+    // register i of block b: channel v0 + b * 32 + (i / 4) * 8 + half * 4 + i % 4 of the lane's column
     const size_t out_at = (size_t)tok * out_row_stride + (size_t)head * hdv;
     bf16_t* op = out + out_at;
     if (gate) {
@@ -306,7 +328,7 @@ attn_biased_kernel(const bf16_t* __restrict__ q, long q_row_stride, const bf16_t
         for (int b = 0; b < NV; ++b)
 #pragma unroll
             for (int i = 0; i < 16; ++i) {
-                const int ch = b * 32 + (i / 4) * 8 + half * 4 + i % 4;
+                const int ch = v0 + b * 32 + (i / 4) * 8 + half * 4 + i % 4;
                 if (ch < hdv) o[b][i] *= 1.0f / (1.0f + __expf(-(float)gp[ch]));
             }
     }
@@ -316,7 +338,7 @@ attn_biased_kernel(const bf16_t* __restrict__ q, long q_row_stride, const bf16_t
         for (int b = 0; b < NV; ++b)
 #pragma unroll
             for (int g4 = 0; g4 < 4; ++g4) {
-                const int ch = b * 32 + g4 * 8 + half * 4;
+                const int ch = v0 + b * 32 + g4 * 8 + half * 4;
                 if (ch + 3 < hdv) {
                     float4 y = make_float4(o[b][g4 * 4] * inv, o[b][g4 * 4 + 1] * inv, o[b][g4 * 4 + 2] * inv, o[b][g4 * 4 + 3] * inv);
                     *reinterpret_cast<float4*>(fp + ch) = y;
@@ -332,7 +354,7 @@ attn_biased_kernel(const bf16_t* __restrict__ q, long q_row_stride, const bf16_t
     for (int b = 0; b < NV; ++b)
 #pragma unroll
         for (int g4 = 0; g4 < 4; ++g4) {
-            const int ch = b * 32 + g4 * 8 + half * 4;
+            const int ch = v0 + b * 32 + g4 * 8 + half * 4;
             if (ch + 3 < hdv) {
                 ab_bf16x4 y;
 #pragma unroll
@@ -351,10 +373,16 @@ static bool ab_sizes_covered(int hd, int hdv) {
     return hd % 16 == 0 && hdv % 4 == 0 && nk >= 2 && nk <= 8 && nv >= 1 && nv <= 4;
 }
 
-// Whether the kernel covers these sizes: query/key heads of 32 to 128 channels in steps of 16, value heads of up to
-// 128 in steps of 4, pages of 16.
+// The wide form: any head size in steps of 16 up to AB_WIDE_MAX_HD channels, any value size in steps of 4.
+constexpr int AB_WIDE_MAX_HD = 1024;
+static bool ab_sizes_covered_wide(int hd, int hdv) {
+    return hd % 16 == 0 && hd >= 32 && hd <= AB_WIDE_MAX_HD && hdv % 4 == 0 && hdv >= 4;
+}
+
+// Whether the kernel covers these sizes: query/key heads of 32 to 1,024 channels in steps of 16, value heads in steps
+// of 4, pages of 16 (up to 128 channels of either with queries in registers, beyond that in the wide form).
 KA_API int ka_attention_biased_supported(int hd, int hdv, int page_size) {
-    return page_size == AB_PAGE && ab_sizes_covered(hd, hdv) ? 1 : 0;
+    return page_size == AB_PAGE && (ab_sizes_covered(hd, hdv) || ab_sizes_covered_wide(hd, hdv)) ? 1 : 0;
 }
 
 KA_API int ka_attention_biased_query_block() { return AB_COLS; }
@@ -371,7 +399,8 @@ KA_API int ka_attention_biased_bf16(const void* q, long q_row_stride, const void
                                     int maps, int values_in_keys, int out_f32, hipStream_t stream) {
     const char* who = "ka_attention_biased_bf16";
     KA_CHECK(n >= 0 && n_blocks >= 0 && H > 0 && Hkv > 0 && H % Hkv == 0, "%s: bad sizes", who);
-    KA_CHECK(page_size == AB_PAGE && ab_sizes_covered(hd, hdv), "%s: head sizes %d / %d or page size %d not covered", who, hd, hdv, page_size);
+    const bool wide = !ab_sizes_covered(hd, hdv);
+    KA_CHECK(page_size == AB_PAGE && (!wide || ab_sizes_covered_wide(hd, hdv)), "%s: head sizes %d / %d or page size %d not covered", who, hd, hdv, page_size);
     KA_CHECK(max_pages > 0, "%s: bad table width %d", who, max_pages);
     KA_CHECK(waves == 4 || waves == 8, "%s: %d waves", who, waves);
     KA_CHECK((uintptr_t)q % 16 == 0 && q_row_stride % 8 == 0 && (uintptr_t)k_cache % 16 == 0,
@@ -398,8 +427,10 @@ KA_API int ka_attention_biased_bf16(const void* q, long q_row_stride, const void
         KA_CHECK(n <= 65535, "%s: too many decode rows %d", who, n);
     }
     KA_CHECK(grid.y <= 65535, "%s: too many blocks %d", who, (int)grid.y);
-    const int nk = hd / 16, nv = (hdv + 31) / 32;
-    const size_t lds = (size_t)(waves / 2) * (16 * nv + 2) * KA_WAVE * sizeof(float);
+    const int nk = wide ? 0 : hd / 16, nv = wide ? 4 : (hdv + 31) / 32;
+    if (wide) grid.z = (hdv + 127) / 128;
+    // the merge area of the waves and, in the wide form, the queries of the 32 columns
+    const size_t lds = (size_t)(waves / 2) * (16 * nv + 2) * KA_WAVE * sizeof(float) + (wide ? (size_t)hd * 32 * sizeof(bf16_t) : 0);
 #define AB_LAUNCH(NK, NV)                                                                                                  \
     if (nk == NK && nv == NV) {                                                                                            \
         static bool sized = false;                                                                                         \
@@ -411,10 +442,11 @@ KA_API int ka_attention_biased_bf16(const void* q, long q_row_stride, const void
                            q_row_stride, (const bf16_t*)k_cache, (const bf16_t*)v_cache, block_table, max_pages, qblk_row, \
                            qblk_tok, cu_q, token_row, kv_lo, kv_hi, positions, slopes, (bf16_t*)out, out_row_stride, scale, \
                            H, Hkv, hdv, heads_per_block, has_sink, sink_score, bias_table, bias_len, (const bf16_t*)gate, \
-                           gate_row_stride, sinks, keep_first, maps, values_in_keys, out_f32);                                                                            \
+                           gate_row_stride, sinks, keep_first, maps, values_in_keys, out_f32, hd);                                                                            \
     }
 #define AB_LAUNCH_NK(NK) AB_LAUNCH(NK, 1) AB_LAUNCH(NK, 2) AB_LAUNCH(NK, 3) AB_LAUNCH(NK, 4)
     AB_LAUNCH_NK(2) AB_LAUNCH_NK(3) AB_LAUNCH_NK(4) AB_LAUNCH_NK(5) AB_LAUNCH_NK(6) AB_LAUNCH_NK(7) AB_LAUNCH_NK(8)
+    AB_LAUNCH(0, 4)
 #undef AB_LAUNCH_NK
 #undef AB_LAUNCH
     KA_LAUNCH_CHECK();
