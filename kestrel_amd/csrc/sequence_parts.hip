@@ -131,10 +131,12 @@ __device__ __forceinline__ float sp_conv_at(const ConvArgs& a, int t, int local,
 }
 
 constexpr int SP_MAX_ROT = 1024;
+constexpr int SP_SPREAD_TOKENS = 128;       // up to this many tokens a step, a token's channels are spread over workgroups
 
-// Grid (tokens, blocks of SP_THREADS channels): a thread per token and channel. The angles of a token are the same for
-// every head: a workgroup computes their cosines and sines once, into LDS. Of a rotated pair of channels the thread of the
-// first computes both convolutions and writes both results.
+// Grid (tokens, workgroups a token): a token's channels are dealt out over its workgroups (a thread per channel in steps
+// of a few tokens, where launches are short and latency counts; one workgroup a token in long steps). The angles of a
+// token are the same for every head: a workgroup computes their cosines and sines once, into LDS. Of a rotated pair of
+// channels the thread of the first computes both convolutions and writes both results.
 template <typename T>
 __global__ void __launch_bounds__(SP_THREADS) conv_prepare_kernel(ConvArgs a) {
     __shared__ float cs[SP_MAX_ROT / 2], sn[SP_MAX_ROT / 2];
@@ -153,16 +155,14 @@ __global__ void __launch_bounds__(SP_THREADS) conv_prepare_kernel(ConvArgs a) {
     }
     T* q_out = reinterpret_cast<T*>(a.q_out) + (size_t)t * a.q_stride;
     T* k_out = reinterpret_cast<T*>(a.k_cache) + ((size_t)page * a.Hk * a.page_size + off) * a.hd;
-    {
-        const int c = blockIdx.y * SP_THREADS + threadIdx.x;
-        if (c >= a.C) return;
+    for (int c = blockIdx.y * SP_THREADS + threadIdx.x; c < a.C; c += gridDim.y * SP_THREADS) {
         if (c < Cq + Ck) {
             const int within = c < Cq ? c : c - Cq;
             const int head = within / a.hd, d = within % a.hd;
             T* dst = c < Cq ? q_out + c : (at >= 0 ? k_out + (size_t)head * a.page_size * a.hd + d : nullptr);
             if (a.freqs && d < a.rot) {
                 const bool first = a.interleaved ? (d & 1) == 0 : d < half;
-                if (!first) return;                     // (written by the thread of its partner)
+                if (!first) continue;                   // (written by the thread of its partner)
                 const int step = a.interleaved ? 1 : half;
                 const int i = a.interleaved ? d / 2 : d;
                 const float y = sp_conv_at<T>(a, t, local, slot, c), other = sp_conv_at<T>(a, t, local, slot, c + step);
@@ -224,8 +224,8 @@ KA_API int ka_conv_prepare(const void* u, int dtype, long u_stride, const float*
     if (n == 0) return 0;
     const int blocks = (a.C + SP_THREADS - 1) / SP_THREADS;
     KA_CHECK(blocks <= 65535, "ka_conv_prepare: too many channels %d", a.C);
-    if (dtype == KA_F32) hipLaunchKernelGGL(conv_prepare_kernel<float>, dim3(n, blocks), dim3(SP_THREADS), 0, stream, a);
-    else hipLaunchKernelGGL(conv_prepare_kernel<bf16_t>, dim3(n, blocks), dim3(SP_THREADS), 0, stream, a);
+    if (dtype == KA_F32) hipLaunchKernelGGL(conv_prepare_kernel<float>, dim3(n, n > SP_SPREAD_TOKENS ? 1 : blocks), dim3(SP_THREADS), 0, stream, a);
+    else hipLaunchKernelGGL(conv_prepare_kernel<bf16_t>, dim3(n, n > SP_SPREAD_TOKENS ? 1 : blocks), dim3(SP_THREADS), 0, stream, a);
     KA_LAUNCH_CHECK();
     if (K > 1 && n_rows > 0) {
         if (dtype == KA_F32) hipLaunchKernelGGL(conv_state_kernel<float>, dim3(n_rows, blocks), dim3(SP_THREADS), 0, stream, a);
