@@ -19,7 +19,9 @@ greedy requests of such a run are compared, token by token, with the plain imple
 feed-forward, heads, head size, runs of layers, vocabulary; random weights): a prompt alone and decode steps at batch 1,
 8 and 64 through the same step function, each with its share of the roofline (``--compare-sizes``, ``--compare-model``).
 ``--workload compare-bogivik`` does the same for the Bogivik design (layers of attention with a distance bias and a
-layer of chunked attention beside a matrix memory) at sizes of its own (``BOGIVIK_SIZES``).
+layer of chunked attention beside a matrix memory) at sizes of its own (``BOGIVIK_SIZES``), and
+``--workload compare-letevik`` for the Letevik design (differential attention behind short convolutions and latent
+attention in a looped stretch of layers; ``LETEVIK_SIZES``).
 """
 
 from __future__ import annotations

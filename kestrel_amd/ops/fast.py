@@ -692,7 +692,8 @@ def attention_maps_bf16(q, k_cache, v_cache, block_table, token_row, kv_lo, kv_h
 
 def attention_latent_bf16(q, cache, block_table, token_row, kv_hi, out, scale, n_heads, row_dim, rank, sinks, batch) -> bool:
     """``n_heads`` query heads of ``row_dim`` channels over one cached row per key whose first ``rank`` channels are its
-    value, with a sink score per head, on the matrix cores. False: not covered (rows above 128 channels among others)."""
+    value, with a sink score per head, on the matrix cores (rows above 128 channels: the kernel's wide form). False: not
+    covered (rows that are no multiple of 16 channels among others)."""
     return attention_biased_bf16(q, cache, None, block_table, token_row, None, kv_hi, out, scale, n_heads, 1, row_dim, rank,
                                  None, None, None, batch, sinks=sinks, values_in_keys=True)
 

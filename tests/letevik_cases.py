@@ -39,7 +39,7 @@ def _config(vocab, width, eps, bigram, layers, loop=None):
 CONFIGS: Dict[str, dict] = {
     # sizes the matrix-core kernels take; a window of one and a half pages that keeps four keys; the loop over the first two layers
     "P": _config(300, 64, 1e-5, (97, 7, 13), [
-        differential(4, 2, 32, 64, 0.2, 0.4, 3, (24, 4), (32, 10000.0), 128, 1.5),
+        differential(4, 2, 32, 64, 0.2, 0.4, 3, (24, 4), (32, 8000.0), 128, 1.5),
         latent(4, 32, 16, 32, 48, 64, 0.15, 50000.0, 128, 3.0),
         differential(2, 2, 64, 32, 0.12, 0.7, 4, (40, 0), (16, 500.0), None),
         latent(2, 64, 32, 64, 32, 128, 0.1, 1e4, 128, 2.0),
@@ -53,10 +53,10 @@ CONFIGS: Dict[str, dict] = {
         differential(3, 1, 28, 36, 0.2, 0.55, 5, (33, 1), (28, 20.0), None),
     ], (1, 3, 3)),
     # no loop at all, one tap (a convolution without state), no convolution, no mask, kept keys beyond a page, a window of whole pages
-    "R": _config(190, 128, 1e-3, (1021, 1, 1), [
+    "R": _config(190, 128, 1e-3, (769, 1, 1), [
         differential(2, 1, 64, 128, 0.09, 0.5, 1, (32, 17), (64, 1e6), 136, 2.0),
         differential(4, 4, 32, 32, 0.18, 0.2, None, None, (8, 1e4), 136, 2.5),
-        latent(8, 64, 16, 64, 128, 96, 0.11, 50000.0, 136, 2.0),
+        latent(8, 48, 16, 64, 96, 80, 0.12, 30000.0, 136, 2.0),
     ]),
     # one of everything: one head, one pass of the loop, a window of one key that keeps one, one bucket
     "S": _config(77, 48, 1e-5, (1, 3, 5), [

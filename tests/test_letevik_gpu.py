@@ -711,7 +711,7 @@ def test_two_maps_on_the_matrix_cores(hd, hdv, window, kept, cut):
 
 @pytest.mark.parametrize("cut", list(_CUTS))
 @pytest.mark.parametrize("heads", [5, 40])
-@pytest.mark.parametrize("rank, dr", [(64, 16), (96, 16), (48, 32), (96, 32), (20, 12), (128, 32), (512, 64), (260, 28)])
+@pytest.mark.parametrize("rank, dr", [(64, 16), (80, 16), (48, 32), (96, 32), (20, 12), (128, 32), (512, 64), (260, 28)])
 def test_latents_with_sinks_on_the_matrix_cores(rank, dr, heads, cut):
     """The bf16 kernel over cached rows that are key and value at once, a sink score per head; in a decode step more heads
     than one workgroup's columns. (Rows above 128 numbers: the kernel's wide form.)"""
@@ -770,7 +770,7 @@ def test_the_matrix_core_kernels_run_where_sizes_allow():
 
 
 @pytest.mark.parametrize("n", [1, 8, 70, 300])
-@pytest.mark.parametrize("heads, a_head, k, out_head, n_out", [(5, 72, 64, 112, 96), (3, 32, 32, 40, 40), (16, 96, 96, 64, 64),
+@pytest.mark.parametrize("heads, a_head, k, out_head, n_out", [(5, 72, 64, 88, 80), (3, 32, 32, 40, 40), (16, 96, 96, 64, 64),
                                                                  (2, 144, 128, 20, 20), (7, 16, 16, 8, 6)])
 def test_a_linear_per_head_on_the_matrix_cores(heads, a_head, k, out_head, n_out, n):
     """Every head's own matrix in one launch: heads that read the first ``k`` channels of their part of a row and write the
