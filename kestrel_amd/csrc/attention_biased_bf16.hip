@@ -24,6 +24,11 @@
 //    and values at once); the value operand is then gathered from the key page;
 //  * out_f32: outputs leave as fp32.
 //
+// A decode step of few rows has few workgroups. With n_splits > 1 a row's tiles of keys are dealt out over that many
+// workgroups in contiguous runs; each leaves its unnormalised outputs, reference point and sum in `partial`
+// (fp32 [tokens, H, n_splits, hdv + 2]), and attn_biased_finish_kernel merges them (the sink, the gate and the
+// output's type are then its business).
+//
 // Heads wider than 128 channels (latent rows of several hundred numbers) take the same loop in its wide form (NK = 0):
 // the head size is a run-time number, the queries of the workgroup's 32 columns lie in LDS instead of registers (every
 // wave reads them from there, 16 bytes a lane and step), keys are streamed step by step, and a workgroup owns a slice of
@@ -79,7 +84,7 @@ attn_biased_kernel(const bf16_t* __restrict__ q, long q_row_stride, const bf16_t
                    long out_row_stride, float scale, int H, int Hkv, int hdv, int heads_per_block, int has_sink,
                    float sink_score, const float* __restrict__ bias_table, int bias_len, const bf16_t* __restrict__ gate,
                    long gate_row_stride, const float* __restrict__ sinks, int keep_first, int maps, int values_in_keys,
-                   int out_f32, int hd_wide) {
+                   int out_f32, int hd_wide, int n_splits, float* __restrict__ partial) {
     constexpr bool WIDE = NK == 0;
     const int HD = WIDE ? hd_wide : NK * 16;
     const int v0 = WIDE ? blockIdx.z * (NV * 32) : 0;     // the first value channel of this workgroup's slice
@@ -91,10 +96,13 @@ attn_biased_kernel(const bf16_t* __restrict__ q, long q_row_stride, const bf16_t
     const int G = H / Hkv;
     int kvh, head, tok, row;
     bool live;
+    int split = 0;
     if (heads_per_block > 1) {
         const int groups = (G + heads_per_block - 1) / heads_per_block;
-        kvh = blockIdx.x / groups;
-        const int hq = (blockIdx.x % groups) * heads_per_block + col;
+        const int bx = blockIdx.x % (Hkv * groups);
+        split = blockIdx.x / (Hkv * groups);
+        kvh = bx / groups;
+        const int hq = (bx % groups) * heads_per_block + col;
         live = col < heads_per_block && hq < G;
         // (maps == 1: head kvh * G + hq)
         head = ((kvh / maps) * G + (live ? hq : 0)) * maps + kvh % maps;
@@ -168,7 +176,9 @@ attn_biased_kernel(const bf16_t* __restrict__ q, long q_row_stride, const bf16_t
         // tiles of kept first keys that lie wholly before the window's first tile come ahead of the window's
         const int kept_tiles = min((min(keep_first, blk_lo) + AB_TILE - 1) / AB_TILE, first_tile);
         const int n_tiles = kept_tiles + last_tile - first_tile + 1;
-        for (int turn = wave; turn < n_tiles; turn += n_waves) {
+        const int per_split = (n_tiles + n_splits - 1) / n_splits;
+        const int turn_end = min(n_tiles, (split + 1) * per_split);
+        for (int turn = split * per_split + wave; turn < turn_end; turn += n_waves) {
             const int tile = turn < kept_tiles ? turn : first_tile + (turn - kept_tiles);
             const int base = tile * AB_TILE;
             // pages of the tile (a page the row has given back, or none: any page, its keys are masked)
@@ -308,6 +318,21 @@ attn_biased_kernel(const bf16_t* __restrict__ q, long q_row_stride, const bf16_t
         __syncthreads();
     }
     if (wave != 0 || !live) return;
+    if (n_splits > 1) {
+        float* pp = partial + (((size_t)tok * H + head) * n_splits + split) * (hdv + 2);
+#pragma unroll
+        for (int b = 0; b < NV; ++b)
+#pragma unroll
+            for (int i = 0; i < 16; ++i) {
+                const int ch = v0 + b * 32 + (i / 4) * 8 + half * 4 + i % 4;
+                if (ch < hdv) pp[ch] = o[b][i];
+            }
+        if (v0 == 0 && half == 0) {
+            pp[hdv] = m;
+            pp[hdv + 1] = l;
+        }
+        return;
+    }
     if (has_sink) {
         const float m_new = fmaxf(m, sink2);
         const float c = __builtin_amdgcn_exp2f(m - m_new);
@@ -368,6 +393,37 @@ attn_biased_kernel(const bf16_t* __restrict__ q, long q_row_stride, const bf16_t
         }
 }
 
+// Merges the partial results of a decode step whose rows' keys were split over workgroups: a wave per (token, head).
+__global__ void __launch_bounds__(KA_WAVE)
+attn_biased_finish_kernel(const float* __restrict__ partial, int n_splits, int H, int hdv, void* __restrict__ out,
+                          long out_row_stride, int out_f32, int has_sink, float sink_score, const float* __restrict__ sinks,
+                          const bf16_t* __restrict__ gate, long gate_row_stride) {
+    const int tok = blockIdx.x, head = blockIdx.y, lane = threadIdx.x;
+    const float* pp = partial + ((size_t)tok * H + head) * n_splits * (hdv + 2);
+    const float sink2 = (sinks ? sinks[head] : sink_score) * AB_LOG2E;
+    float top = has_sink ? sink2 : -INFINITY;
+    for (int s = 0; s < n_splits; ++s) top = fmaxf(top, pp[(size_t)s * (hdv + 2) + hdv]);
+    float total = has_sink ? __builtin_amdgcn_exp2f(sink2 - top) : 0.f;
+    for (int s = 0; s < n_splits; ++s) {
+        const float ms = pp[(size_t)s * (hdv + 2) + hdv], ls = pp[(size_t)s * (hdv + 2) + hdv + 1];
+        if (ls > 0.f) total += ls * __builtin_amdgcn_exp2f(ms - top);
+    }
+    const float inv = total > 0.f ? 1.0f / total : 0.f;
+    const size_t out_at = (size_t)tok * out_row_stride + (size_t)head * hdv;
+    for (int ch = lane; ch < hdv; ch += KA_WAVE) {
+        float acc = 0.f;
+        for (int s = 0; s < n_splits; ++s) {
+            const float ls = pp[(size_t)s * (hdv + 2) + hdv + 1];
+            // (a split that saw no key left nothing to add, and its outputs may be anything)
+            if (ls > 0.f) acc += pp[(size_t)s * (hdv + 2) + ch] * __builtin_amdgcn_exp2f(pp[(size_t)s * (hdv + 2) + hdv] - top);
+        }
+        float y = acc * inv;
+        if (gate) y *= 1.0f / (1.0f + __expf(-(float)gate[(size_t)tok * gate_row_stride + (size_t)head * hdv + ch]));
+        if (out_f32) reinterpret_cast<float*>(out)[out_at + ch] = y;
+        else reinterpret_cast<bf16_t*>(out)[out_at + ch] = (bf16_t)y;
+    }
+}
+
 static bool ab_sizes_covered(int hd, int hdv) {
     const int nk = hd / 16, nv = (hdv + 31) / 32;
     return hd % 16 == 0 && hdv % 4 == 0 && nk >= 2 && nk <= 8 && nv >= 1 && nv <= 4;
@@ -396,7 +452,8 @@ KA_API int ka_attention_biased_bf16(const void* q, long q_row_stride, const void
                                     long out_row_stride, float scale, int n, int H, int Hkv, int hd, int hdv,
                                     int page_size, int waves, int has_sink, float sink_score, const float* bias_table,
                                     int bias_len, const void* gate, long gate_row_stride, const float* sinks, int keep_first,
-                                    int maps, int values_in_keys, int out_f32, hipStream_t stream) {
+                                    int maps, int values_in_keys, int out_f32, int n_splits, float* partial,
+                                    hipStream_t stream) {
     const char* who = "ka_attention_biased_bf16";
     KA_CHECK(n >= 0 && n_blocks >= 0 && H > 0 && Hkv > 0 && H % Hkv == 0, "%s: bad sizes", who);
     const bool wide = !ab_sizes_covered(hd, hdv);
@@ -414,6 +471,8 @@ KA_API int ka_attention_biased_bf16(const void* q, long q_row_stride, const void
     KA_CHECK(slopes == nullptr || positions != nullptr, "%s: slopes need the queries' positions", who);
     KA_CHECK(bias_table == nullptr || (positions != nullptr && bias_len > 0), "%s: a distance table needs the queries' positions", who);
     KA_CHECK(n_blocks == 0 || (qblk_row && qblk_tok && cu_q), "%s: blocks of queries need their lists", who);
+    KA_CHECK(n_splits >= 1 && n_splits <= 64 && (n_splits == 1 || (n_blocks == 0 && partial != nullptr)),
+             "%s: %d splits (keys are split in decode steps only, and need room for the partial results)", who, n_splits);
     if (n == 0) return 0;
     const int G = H / Hkv;
     int heads_per_block = 1;
@@ -423,7 +482,7 @@ KA_API int ka_attention_biased_bf16(const void* q, long q_row_stride, const void
     } else {
         // (with a single query head per kv head the columns hold one query: heads_per_block 1 would mean blocks)
         heads_per_block = G < 2 ? 2 : (G > AB_COLS ? AB_COLS : G);
-        grid = dim3(Hkv * ((G + heads_per_block - 1) / heads_per_block), n);
+        grid = dim3(Hkv * ((G + heads_per_block - 1) / heads_per_block) * n_splits, n);
         KA_CHECK(n <= 65535, "%s: too many decode rows %d", who, n);
     }
     KA_CHECK(grid.y <= 65535, "%s: too many blocks %d", who, (int)grid.y);
@@ -442,7 +501,7 @@ KA_API int ka_attention_biased_bf16(const void* q, long q_row_stride, const void
                            q_row_stride, (const bf16_t*)k_cache, (const bf16_t*)v_cache, block_table, max_pages, qblk_row, \
                            qblk_tok, cu_q, token_row, kv_lo, kv_hi, positions, slopes, (bf16_t*)out, out_row_stride, scale, \
                            H, Hkv, hdv, heads_per_block, has_sink, sink_score, bias_table, bias_len, (const bf16_t*)gate, \
-                           gate_row_stride, sinks, keep_first, maps, values_in_keys, out_f32, hd);                                                                            \
+                           gate_row_stride, sinks, keep_first, maps, values_in_keys, out_f32, hd, n_splits, partial);                                                                            \
     }
 #define AB_LAUNCH_NK(NK) AB_LAUNCH(NK, 1) AB_LAUNCH(NK, 2) AB_LAUNCH(NK, 3) AB_LAUNCH(NK, 4)
     AB_LAUNCH_NK(2) AB_LAUNCH_NK(3) AB_LAUNCH_NK(4) AB_LAUNCH_NK(5) AB_LAUNCH_NK(6) AB_LAUNCH_NK(7) AB_LAUNCH_NK(8)
@@ -450,5 +509,11 @@ KA_API int ka_attention_biased_bf16(const void* q, long q_row_stride, const void
 #undef AB_LAUNCH_NK
 #undef AB_LAUNCH
     KA_LAUNCH_CHECK();
+    if (n_splits > 1) {
+        KA_CHECK(H <= 65535, "%s: too many heads %d", who, H);
+        hipLaunchKernelGGL(attn_biased_finish_kernel, dim3(n, H), dim3(KA_WAVE), 0, stream, partial, n_splits, H, hdv, out,
+                           out_row_stride, out_f32, has_sink, sink_score, sinks, (const bf16_t*)gate, gate_row_stride);
+        KA_LAUNCH_CHECK();
+    }
     return 0;
 }

@@ -58,7 +58,7 @@ _SIGNATURES = {
     "ka_attention_biased_bf16": [_c_void_p, _c_long, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_void_p, _c_void_p, _c_int,
                                  _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_long, _c_float,
                                  _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_void_p, _c_int, _c_void_p, _c_long,
-                                 _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_void_p],
+                                 _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void_p, _c_void_p],
     "ka_heads_linear_bf16": [_c_void_p, _c_long, _c_int, _c_void_p, _c_void_p, _c_long, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void_p,
                              _c_long, _c_void_p],
     "ka_heads_linear_supported": [_c_long, _c_int, _c_long, _c_int, _c_int, _c_int],
@@ -80,6 +80,9 @@ NORM_AFTER_MAX_WIDTH = 8192
 # the persistent kernel then repeats the LayerNorm of all rows once; with a few hundred workgroups
 # that is cheaper than a launch of its own (measured on MI355X: 3 % of a decode step at batch 8).
 FUSE_LAYERNORM_PROLOGUE = True
+# Whether the matrix-core attention with further terms deals a row's keys out over several workgroups in decode steps
+# of few rows (``attention_biased_bf16``).
+SPLIT_DECODE_KEYS = True
 # Whether the decode attention of a few rows (whose workgroups fill at most a quarter of the chip)
 # takes the feed-forward's first linear into its own launch instead of leaving it to the launch of
 # the q|k|v projection before it (measured on MI355X at Moondream 2's sizes: 3 to 5 % of a decode
@@ -653,12 +656,22 @@ def attention_biased_bf16(q, k_cache, v_cache, block_table, token_row, kv_lo, kv
     if bias_table is not None and (bias_table.dtype != torch.float32 or bias_table.dim() != 2 or bias_table.shape[0] != n_heads
                                    or not bias_table.is_contiguous() or positions is None):
         raise KernelError("attention: the distance table must be contiguous fp32 [H, T] and come with the queries' positions")
+    n_splits, partial = 1, None
     if batch.decode_only:
         rows = first = None
         n_blocks = 0
         groups = n_heads // n_kv_heads
         workgroups = n * n_kv_heads * -(-groups // 32)
         waves = 4 if workgroups >= 2 * chip_sizes(q.device).compute_units else 8
+        # few rows: a row's keys are dealt out over several workgroups, whose partial results a second launch merges
+        # (the number depends on the rows alone, so a captured step keeps its layout)
+        units = chip_sizes(q.device).compute_units
+        scratch_of = getattr(batch, "workspace", None)
+        # (measured on MI355X: with more than an eighth of the chip's units busy, or more than four runs of keys a row,
+        # the second launch costs more than the split gains)
+        if SPLIT_DECODE_KEYS and scratch_of is not None and 8 * workgroups <= units:
+            n_splits = 4
+            partial = scratch_of.get("attention.partials", (n, n_heads, n_splits, value_dim + 2), torch.float32)
     else:
         size = int(handle.ka_attention_biased_query_block())
         listed = (getattr(batch, "query_blocks", None) or {}).get(size)
@@ -678,7 +691,7 @@ def attention_biased_bf16(q, k_cache, v_cache, block_table, token_row, kv_lo, kv
         value_dim, page_size, waves, int(sink is not None or sinks is not None), float(sink or 0.0), _ptr(bias_table),
         int(bias_table.shape[1]) if bias_table is not None else 0, _ptr(gate),
         (gate.stride(0) if n > 1 else n_heads * value_dim) if gate is not None else 0, _ptr(sinks), int(keep_first), int(maps),
-        int(bool(values_in_keys)), int(out_f32), stream_ptr()))
+        int(bool(values_in_keys)), int(out_f32), n_splits, _ptr(partial), stream_ptr()))
     return True
 
 

@@ -656,8 +656,12 @@ class _Packed:
         self.token_row, self.kv_hi, self.cu_q = _i32(token_row), _i32(kv_hi), _i32(cu_q)
         self.kv_lo = _i32(kv_lo) if window is not None else None
         self.table = table.to(DEV)
+        from kestrel_amd.engine.batch import Workspace
+
+        # (with a workspace at hand a decode step of few rows deals a row's keys out over several workgroups)
         self.batch = SimpleNamespace(decode_only=all(n - s == 1 for n, s in zip(lengths, starts)),
-                                     query_blocks={32: (_i32(rows), _i32(first))}, cu_q=self.cu_q)
+                                     query_blocks={32: (_i32(rows), _i32(first))}, cu_q=self.cu_q,
+                                     workspace=Workspace(torch.device(DEV)))
 
     def pages(self, per_row, transposed=False):
         """``per_row[r]`` ``[length, heads, channels]`` into pages ``[pages, heads, 16, channels]`` (or ``[pages, heads, channels, 16]``);
