@@ -22,7 +22,9 @@
 //    Hkv / maps heads);
 //  * values_in_keys: a key's value is the first hdv channels of its key row (a cache of latents that are keys
 //    and values at once); the value operand is then gathered from the key page;
-//  * out_f32: outputs leave as fp32.
+//  * out_f32: outputs leave as fp32;
+//  * softcap > 0: scale * (q . k) passes through softcap * tanh(. / softcap) before the other terms are added;
+//  * gate_per_head: the output gate holds one number per head ([n, H]) instead of one per channel.
 //
 // A decode step of few rows has few workgroups. With n_splits > 1 a row's tiles of keys are dealt out over that many
 // workgroups in contiguous runs; each leaves its unnormalised outputs, reference point and sum in `partial`
@@ -84,7 +86,7 @@ attn_biased_kernel(const bf16_t* __restrict__ q, long q_row_stride, const bf16_t
                    long out_row_stride, float scale, int H, int Hkv, int hdv, int heads_per_block, int has_sink,
                    float sink_score, const float* __restrict__ bias_table, int bias_len, const bf16_t* __restrict__ gate,
                    long gate_row_stride, const float* __restrict__ sinks, int keep_first, int maps, int values_in_keys,
-                   int out_f32, int hd_wide, int n_splits, float* __restrict__ partial) {
+                   int out_f32, int hd_wide, int n_splits, float* __restrict__ partial, float softcap, int gate_per_head) {
     constexpr bool WIDE = NK == 0;
     const int HD = WIDE ? hd_wide : NK * 16;
     const int v0 = WIDE ? blockIdx.z * (NV * 32) : 0;     // the first value channel of this workgroup's slice
@@ -145,7 +147,9 @@ attn_biased_kernel(const bf16_t* __restrict__ q, long q_row_stride, const bf16_t
         }
     }
     const float slope2 = slopes ? slopes[head] * AB_LOG2E : 0.f;     // in powers of two, like everything below
-    const float scale2 = scale * AB_LOG2E;
+    // (a cap: the product is first brought to score / cap, whose tanh times cap, in powers of two, is the score)
+    const float scale2 = softcap > 0.f ? scale / softcap * (2.0f * AB_LOG2E) : scale * AB_LOG2E;
+    const float cap2 = softcap * AB_LOG2E;
     const int place = (slopes || bias_table) ? positions[tok] : 0;
     const float* bias_row = bias_table ? bias_table + (size_t)head * bias_len : nullptr;
     const float bias_far2 = bias_row ? bias_row[bias_len - 1] * AB_LOG2E : 0.f;
@@ -250,7 +254,14 @@ attn_biased_kernel(const bf16_t* __restrict__ q, long q_row_stride, const bf16_t
 #pragma unroll
             for (int i = 0; i < 16; ++i) {
                 const int off = (i / 8) * 16 + i % 8;
-                float x = fmaf(s[i], scale2, fmaf(slope2, (float)off, bias0));
+                float x;
+                if (softcap > 0.f) {
+                    // tanh(z) = 1 - 2 / (e^(2z) + 1), with s * scale2 = 2 z log2(e)
+                    const float e = __builtin_amdgcn_exp2f(s[i] * scale2);
+                    x = fmaf(cap2, 1.0f - 2.0f * __builtin_amdgcn_rcpf(e + 1.0f), fmaf(slope2, (float)off, bias0));
+                } else {
+                    x = fmaf(s[i], scale2, fmaf(slope2, (float)off, bias0));
+                }
                 if (near_tile) x = fmaf(bias_row[min(max(place - (j0 + off), 0), bias_len - 1)], AB_LOG2E, x);
                 else x += bias_far2;
                 if (!whole) {
@@ -346,7 +357,13 @@ attn_biased_kernel(const bf16_t* __restrict__ q, long q_row_stride, const bf16_t
     // register i of block b: channel v0 + b * 32 + (i / 4) * 8 + half * 4 + i % 4 of the lane's column
     const size_t out_at = (size_t)tok * out_row_stride + (size_t)head * hdv;
     bf16_t* op = out + out_at;
-    if (gate) {
+    if (gate && gate_per_head) {
+        const float y = 1.0f / (1.0f + __expf(-(float)gate[(size_t)tok * gate_row_stride + head]));
+#pragma unroll
+        for (int b = 0; b < NV; ++b)
+#pragma unroll
+            for (int i = 0; i < 16; ++i) o[b][i] *= y;
+    } else if (gate) {
         // an output gate: every channel times the sigmoid of the gate's pre-activation of the same token and channel
         const bf16_t* gp = gate + (size_t)tok * gate_row_stride + (size_t)head * hdv;
 #pragma unroll
@@ -397,7 +414,7 @@ attn_biased_kernel(const bf16_t* __restrict__ q, long q_row_stride, const bf16_t
 __global__ void __launch_bounds__(KA_WAVE)
 attn_biased_finish_kernel(const float* __restrict__ partial, int n_splits, int H, int hdv, void* __restrict__ out,
                           long out_row_stride, int out_f32, int has_sink, float sink_score, const float* __restrict__ sinks,
-                          const bf16_t* __restrict__ gate, long gate_row_stride) {
+                          const bf16_t* __restrict__ gate, long gate_row_stride, int gate_per_head) {
     const int tok = blockIdx.x, head = blockIdx.y, lane = threadIdx.x;
     const float* pp = partial + ((size_t)tok * H + head) * n_splits * (hdv + 2);
     const float sink2 = (sinks ? sinks[head] : sink_score) * AB_LOG2E;
@@ -418,7 +435,7 @@ attn_biased_finish_kernel(const float* __restrict__ partial, int n_splits, int H
             if (ls > 0.f) acc += pp[(size_t)s * (hdv + 2) + ch] * __builtin_amdgcn_exp2f(pp[(size_t)s * (hdv + 2) + hdv] - top);
         }
         float y = acc * inv;
-        if (gate) y *= 1.0f / (1.0f + __expf(-(float)gate[(size_t)tok * gate_row_stride + (size_t)head * hdv + ch]));
+        if (gate) y *= 1.0f / (1.0f + __expf(-(float)gate[(size_t)tok * gate_row_stride + (gate_per_head ? (size_t)head : (size_t)head * hdv + ch)]));
         if (out_f32) reinterpret_cast<float*>(out)[out_at + ch] = y;
         else reinterpret_cast<bf16_t*>(out)[out_at + ch] = (bf16_t)y;
     }
@@ -453,8 +470,9 @@ KA_API int ka_attention_biased_bf16(const void* q, long q_row_stride, const void
                                     int page_size, int waves, int has_sink, float sink_score, const float* bias_table,
                                     int bias_len, const void* gate, long gate_row_stride, const float* sinks, int keep_first,
                                     int maps, int values_in_keys, int out_f32, int n_splits, float* partial,
-                                    hipStream_t stream) {
+                                    float softcap, int gate_per_head, hipStream_t stream) {
     const char* who = "ka_attention_biased_bf16";
+    KA_CHECK(softcap >= 0.f, "%s: a cap on the scores must be positive", who);
     KA_CHECK(n >= 0 && n_blocks >= 0 && H > 0 && Hkv > 0 && H % Hkv == 0, "%s: bad sizes", who);
     const bool wide = !ab_sizes_covered(hd, hdv);
     KA_CHECK(page_size == AB_PAGE && (!wide || ab_sizes_covered_wide(hd, hdv)), "%s: head sizes %d / %d or page size %d not covered", who, hd, hdv, page_size);
@@ -501,7 +519,7 @@ KA_API int ka_attention_biased_bf16(const void* q, long q_row_stride, const void
                            q_row_stride, (const bf16_t*)k_cache, (const bf16_t*)v_cache, block_table, max_pages, qblk_row, \
                            qblk_tok, cu_q, token_row, kv_lo, kv_hi, positions, slopes, (bf16_t*)out, out_row_stride, scale, \
                            H, Hkv, hdv, heads_per_block, has_sink, sink_score, bias_table, bias_len, (const bf16_t*)gate, \
-                           gate_row_stride, sinks, keep_first, maps, values_in_keys, out_f32, hd, n_splits, partial);                                                                            \
+                           gate_row_stride, sinks, keep_first, maps, values_in_keys, out_f32, hd, n_splits, partial, softcap, gate_per_head); \
     }
 #define AB_LAUNCH_NK(NK) AB_LAUNCH(NK, 1) AB_LAUNCH(NK, 2) AB_LAUNCH(NK, 3) AB_LAUNCH(NK, 4)
     AB_LAUNCH_NK(2) AB_LAUNCH_NK(3) AB_LAUNCH_NK(4) AB_LAUNCH_NK(5) AB_LAUNCH_NK(6) AB_LAUNCH_NK(7) AB_LAUNCH_NK(8)
@@ -512,7 +530,7 @@ KA_API int ka_attention_biased_bf16(const void* q, long q_row_stride, const void
     if (n_splits > 1) {
         KA_CHECK(H <= 65535, "%s: too many heads %d", who, H);
         hipLaunchKernelGGL(attn_biased_finish_kernel, dim3(n, H), dim3(KA_WAVE), 0, stream, partial, n_splits, H, hdv, out,
-                           out_row_stride, out_f32, has_sink, sink_score, sinks, (const bf16_t*)gate, gate_row_stride);
+                           out_row_stride, out_f32, has_sink, sink_score, sinks, (const bf16_t*)gate, gate_row_stride, gate_per_head);
         KA_LAUNCH_CHECK();
     }
     return 0;

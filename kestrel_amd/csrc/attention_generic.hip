@@ -27,7 +27,9 @@
 //    the value cache has Hkv / maps heads;
 //  * values inside the keys (values_in_keys != 0): the value of a key is the first hdv channels of its key row
 //    (a cache of latents that are both); v_cache is then not read;
-//  * out_f32 != 0: the output is written as fp32 whatever the type of queries and cache.
+//  * out_f32 != 0: the output is written as fp32 whatever the type of queries and cache;
+//  * softcap > 0: the scaled score passes through softcap * tanh(score / softcap) before any bias and the softmax;
+//  * gate_per_head != 0: the gate holds one number per head ([n, H]) instead of one per channel.
 #include "ka_common.h"
 
 constexpr int ATT_MAX_HD = 1024;
@@ -52,7 +54,7 @@ attention_generic_kernel(const T* __restrict__ q, long q_row_stride, const T* __
                          const float* __restrict__ slopes, int has_sink, float sink_score,
                          const float* __restrict__ bias_table, int bias_len, const T* __restrict__ gate,
                          long gate_row_stride, const float* __restrict__ sinks, int keep_first, int maps,
-                         int values_in_keys, int out_f32) {
+                         int values_in_keys, int out_f32, float softcap, int gate_per_head) {
     __shared__ float qs[ATT_MAX_HD];
     __shared__ float ps[KA_WAVE];
     __shared__ long offs[KA_WAVE];   // value cache offset of channel 0 of each key of the chunk
@@ -101,6 +103,7 @@ attention_generic_kernel(const T* __restrict__ q, long q_row_stride, const T* __
             } else {
                 for (int d = 0; d < hd; ++d) acc = fmaf(qs[d], ka_to_float(kp[d]), acc);
             }
+            if (softcap > 0.f) acc = softcap * tanhf(acc / softcap);
             s = slopes ? acc - slope * (float)(place - key) : acc;
             if (bias_row) s += bias_row[min(max(place - key, 0), bias_len - 1)];
         }
@@ -139,13 +142,14 @@ attention_generic_kernel(const T* __restrict__ q, long q_row_stride, const T* __
     }
     float inv = l > 0.f ? 1.0f / l : 0.f;
     const size_t out_at = (size_t)t * out_row_stride + (size_t)h * hdv;
+    const float head_gate = gate && gate_per_head ? 1.0f / (1.0f + expf(-ka_to_float(gate[(size_t)t * gate_row_stride + h]))) : 1.f;
 #pragma unroll
     for (int i = 0; i < ATT_MAX_HD / KA_WAVE; ++i) {
         int d = lane + i * KA_WAVE;
         if (d < hdv) {
-            float y = o[i] * inv;
+            float y = o[i] * inv * head_gate;
             // (an output gate: the head's channels times the sigmoid of the gate's pre-activations of the same token)
-            if (gate) y *= 1.0f / (1.0f + expf(-ka_to_float(gate[(size_t)t * gate_row_stride + (size_t)h * hdv + d])));
+            if (gate && !gate_per_head) y *= 1.0f / (1.0f + expf(-ka_to_float(gate[(size_t)t * gate_row_stride + (size_t)h * hdv + d])));
             if (out_f32) reinterpret_cast<float*>(out)[out_at + d] = y;
             else out[out_at + d] = ka_from_float<T>(y);
         }
@@ -159,7 +163,8 @@ KA_API int ka_attention_generic(const void* q, int dtype, long q_row_stride, con
                                 int page_size, int hdv, const int* positions, const float* slopes,
                                 int has_sink, float sink_score, const float* bias_table, int bias_len,
                                 const void* gate, long gate_row_stride, const float* sinks, int keep_first, int maps,
-                                int values_in_keys, int out_f32, hipStream_t stream) {
+                                int values_in_keys, int out_f32, float softcap, int gate_per_head, hipStream_t stream) {
+    KA_CHECK(softcap >= 0.f, "ka_attention_generic: a cap on the scores must be positive");
     KA_CHECK(maps >= 1 && H % maps == 0 && Hkv % maps == 0 && keep_first >= 0, "ka_attention_generic: %d maps do not divide the heads %d and %d", maps, H, Hkv);
     KA_CHECK(!values_in_keys || hdv <= hd, "ka_attention_generic: values inside keys of %d channels cannot have %d", hd, hdv);
     KA_CHECK(sinks == nullptr || has_sink, "ka_attention_generic: sink scores without a sink");
@@ -177,12 +182,12 @@ KA_API int ka_attention_generic(const void* q, int dtype, long q_row_stride, con
         hipLaunchKernelGGL(attention_generic_kernel<float>, grid, block, 0, stream, (const float*)q, q_row_stride,
                            (const float*)k_cache, (const float*)v_cache, block_table, max_pages, token_row, kv_lo,
                            kv_hi, (float*)out, out_row_stride, scale, H, Hkv, hd, hdv, page_size, positions, slopes, has_sink,
-                           sink_score, bias_table, bias_len, (const float*)gate, gate_row_stride, sinks, keep_first, maps, values_in_keys, out_f32);
+                           sink_score, bias_table, bias_len, (const float*)gate, gate_row_stride, sinks, keep_first, maps, values_in_keys, out_f32, softcap, gate_per_head);
     else if (dtype == KA_BF16)
         hipLaunchKernelGGL(attention_generic_kernel<bf16_t>, grid, block, 0, stream, (const bf16_t*)q, q_row_stride,
                            (const bf16_t*)k_cache, (const bf16_t*)v_cache, block_table, max_pages, token_row, kv_lo,
                            kv_hi, (bf16_t*)out, out_row_stride, scale, H, Hkv, hd, hdv, page_size, positions, slopes, has_sink,
-                           sink_score, bias_table, bias_len, (const bf16_t*)gate, gate_row_stride, sinks, keep_first, maps, values_in_keys, out_f32);
+                           sink_score, bias_table, bias_len, (const bf16_t*)gate, gate_row_stride, sinks, keep_first, maps, values_in_keys, out_f32, softcap, gate_per_head);
     else
         KA_CHECK(false, "ka_attention_generic: unsupported dtype %d", dtype);
     KA_LAUNCH_CHECK();

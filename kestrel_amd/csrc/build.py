@@ -29,7 +29,8 @@ ARCH = "gfx950"
 # library name -> its sources. "core" is all a float32 run needs; "fast" holds the
 # bf16 MFMA kernels of serving.
 LIBRARIES: Dict[str, List[str]] = {
-    "core": ["ka_error.hip", "elementwise.hip", "gemm_generic.hip", "attention_generic.hip", "mixer_parts.hip", "sequence_parts.hip", "sampling.hip", "peaks.hip"],
+    "core": ["ka_error.hip", "elementwise.hip", "gemm_generic.hip", "attention_generic.hip", "mixer_parts.hip", "sequence_parts.hip", "recurrent_parts.hip", "experts.hip",
+             "sampling.hip", "peaks.hip"],
     "fast": ["ka_error.hip", "gemm_bf16.hip", "gemv_bf16.hip", "attention_bf16.hip", "attention_biased_bf16.hip", "heads_linear_bf16.hip", "matrix_memory_bf16.hip", "decode_beside.hip",
              "gemm_library.hip"],
 }

@@ -152,7 +152,7 @@ __device__ __forceinline__ float ka_gelu_tanh_fast(float x) {
 // Activations a linear kernel can apply in its epilogue. One table for every kernel family: a
 // further activation is a code here, a case in each of the two functions below, and its name in
 // the table of the Python face (ops/linear.py).
-enum KaAct : int { KA_ACT_NONE = 0, KA_ACT_GELU_TANH = 1, KA_ACT_RELU = 2, KA_ACT_SILU = 3, KA_ACT_RELU_SQUARED = 4, KA_ACT_COUNT = 5 };
+enum KaAct : int { KA_ACT_NONE = 0, KA_ACT_GELU_TANH = 1, KA_ACT_RELU = 2, KA_ACT_SILU = 3, KA_ACT_RELU_SQUARED = 4, KA_ACT_TANH = 5, KA_ACT_COUNT = 6 };
 
 // A gated linear layer (the first half of a feed-forward of the form act(x Wg^T) * (x Wu^T)): KA_ACT_GATED
 // added to an activation's code says that the rows of the weights come in pairs, row 2j the gate's and
@@ -175,6 +175,7 @@ __device__ __forceinline__ float ka_activate(int act, float x) {
         case KA_ACT_RELU: return fmaxf(x, 0.f);
         case KA_ACT_SILU: return x / (1.0f + expf(-x));
         case KA_ACT_RELU_SQUARED: { const float r = fmaxf(x, 0.f); return r * r; }
+        case KA_ACT_TANH: return tanhf(x);
         default: return x;
     }
 }
@@ -186,6 +187,7 @@ __device__ __forceinline__ float ka_activate_fast(int act, float x) {
         case KA_ACT_RELU: return fmaxf(x, 0.f);
         case KA_ACT_SILU: return x * __fdividef(1.0f, 1.0f + __expf(-x));
         case KA_ACT_RELU_SQUARED: { const float r = fmaxf(x, 0.f); return r * r; }
+        case KA_ACT_TANH: return tanhf(x);
         default: return x;
     }
 }

@@ -66,7 +66,9 @@ KA_API int ka_rmsnorm(const float* x, const int* rows, const float* gain, float 
 //  * values: blend 1 copies them to `v_other` (the values of this layer for later ones), blend 2 replaces them by
 //    (1 - lambda) v + lambda v_other with the fp32 scalar at `lambda`;
 //  * queries go back in place; keys go into the paged cache [pages, G, page_size, hd] (the row keeps them as projected),
-//    values into [pages, G, hdv, page_size] (slots[t] = page * page_size + offset, negative or no slots: nothing is cached).
+//    values into [pages, G, hdv, page_size] (slots[t] = page * page_size + offset, negative or no slots: nothing is cached);
+//  * v_from_k != 0: there are no value columns, the values are the keys as projected (hdv = hd; the row is
+//    [H hd | G hd]); G = 0: a row of queries alone (a layer that reads another layer's keys and values).
 // ----------------------------------------------------------------------------
 struct PrepareArgs {
     void* qkv;
@@ -88,6 +90,7 @@ struct PrepareArgs {
     void* v_other;
     long v_other_stride;
     const float* lambda;
+    int v_from_k;
 };
 
 template <typename T>
@@ -160,7 +163,7 @@ __global__ void __launch_bounds__(MP_THREADS) qkv_prepare_kernel(PrepareArgs a) 
         for (int c = a.rot + lane; c < hd; c += KA_WAVE)
             dst[c] = ka_from_float<T>(ka_to_float(hp[c]) * r * (gain ? gain[c] : 1.f) * after);
     }
-    T* vrow = row + (size_t)heads * hd;
+    T* vrow = row + (size_t)(a.v_from_k ? a.H : heads) * hd;
     const float lam = a.blend == 2 ? *a.lambda : 0.f;
     T* other = a.blend ? reinterpret_cast<T*>(a.v_other) + (size_t)t * a.v_other_stride : nullptr;
     for (int g = wave; g < a.G; g += MP_WAVES)
@@ -262,7 +265,7 @@ __global__ void __launch_bounds__(MP_THREADS) qkv_prepare_wide_kernel(PrepareArg
         for (int u = 0; u < 8; ++u) o[u] = (bf16_t)(y[u] * after);
         *reinterpret_cast<mp_bf16x8*>(dst) = o;
     }
-    bf16_t* vrow = row + (size_t)heads * HD;
+    bf16_t* vrow = row + (size_t)(a.v_from_k ? a.H : heads) * HD;
     const int pieces = a.hdv / 8;
     const float lam = a.blend == 2 ? *a.lambda : 0.f;
     bf16_t* other = a.blend ? reinterpret_cast<bf16_t*>(a.v_other) + (size_t)t * a.v_other_stride : nullptr;
@@ -288,10 +291,12 @@ KA_API int ka_qkv_prepare(void* qkv, int dtype, long row_stride, const int* posi
                           void* v_cache, int n, int H, int G, int hd, int hdv, int page_size, int norm_mode,
                           const float* q_gain, const float* k_gain, float eps, const float* freqs, int rot, int interleaved,
                           float q_coef, int q_every, int blend, void* v_other, long v_other_stride, const float* lambda,
-                          hipStream_t stream) {
+                          int v_from_k, hipStream_t stream) {
     const char* who = "ka_qkv_prepare";
-    KA_CHECK(n >= 0 && H > 0 && G > 0 && hd > 0 && hdv > 0 && page_size > 0, "%s: bad sizes", who);
-    KA_CHECK(row_stride >= (long)(H + G) * hd + (long)G * hdv, "%s: row stride %ld too small", who, row_stride);
+    KA_CHECK(n >= 0 && H > 0 && G >= 0 && hd > 0 && hdv > 0 && page_size > 0, "%s: bad sizes", who);
+    KA_CHECK(!v_from_k || (hdv == hd && blend == 0), "%s: values that are the keys have the keys' size and are not blended", who);
+    KA_CHECK(G > 0 || slots == nullptr, "%s: a row of queries alone caches nothing", who);
+    KA_CHECK(row_stride >= (long)(H + G) * hd + (v_from_k ? 0 : (long)G * hdv), "%s: row stride %ld too small", who, row_stride);
     KA_CHECK(norm_mode >= 0 && norm_mode <= 2 && eps >= 0.f, "%s: norm mode %d", who, norm_mode);
     KA_CHECK(freqs == nullptr || (rot > 0 && rot <= hd && rot % 2 == 0), "%s: %d rotated channels of %d", who, rot, hd);
     KA_CHECK(freqs == nullptr || positions != nullptr, "%s: a rotation needs the tokens' places", who);
@@ -307,7 +312,7 @@ KA_API int ka_qkv_prepare(void* qkv, int dtype, long row_stride, const int* posi
     const size_t lds = ((size_t)(H + G) + rot) * sizeof(float);
     KA_CHECK(lds <= 64 * 1024, "%s: %d heads and %d rotated channels do not fit in LDS", who, H + G, rot);
     PrepareArgs a{qkv, row_stride, positions, slots, k_cache, v_cache, H, G, hd, hdv, page_size, norm_mode, q_gain, k_gain, eps,
-                  freqs, rot, interleaved, q_coef, q_every, blend, v_other, v_other_stride, lambda};
+                  freqs, rot, interleaved, q_coef, q_every, blend, v_other, v_other_stride, lambda, v_from_k};
     // bf16 heads of 32, 64 or 128 channels, everything 16-byte aligned, pairs of neighbours if rotated: eight channels a lane
     const bool wide = dtype == KA_BF16 && (hd == 32 || hd == 64 || hd == 128) && hdv % 8 == 0 && row_stride % 8 == 0 &&
         (uintptr_t)qkv % 16 == 0 && (freqs == nullptr || interleaved == 1) &&

@@ -32,11 +32,11 @@ _SIGNATURES = {
     "ka_attention_generic": [_c_void_p, _c_int, _c_long, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_void_p,
                              _c_void_p, _c_void_p, _c_void_p, _c_long, _c_float, _c_int, _c_int, _c_int, _c_int,
                              _c_int, _c_int, _c_void_p, _c_void_p, _c_int, _c_float, _c_void_p, _c_int, _c_void_p, _c_long,
-                             _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_void_p],
+                             _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _c_void_p],
     "ka_rmsnorm": [_c_void_p, _c_void_p, _c_void_p, _c_float, _c_void_p, _c_int, _c_int, _c_int, _c_void_p],
     "ka_qkv_prepare": [_c_void_p, _c_int, _c_long, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int,
                        _c_int, _c_int, _c_int, _c_void_p, _c_void_p, _c_float, _c_void_p, _c_int, _c_int, _c_float, _c_int,
-                       _c_int, _c_void_p, _c_long, _c_void_p, _c_void_p],
+                       _c_int, _c_void_p, _c_long, _c_void_p, _c_int, _c_void_p],
     "ka_gated_pairs": [_c_void_p, _c_long, _c_void_p, _c_long, _c_int, _c_int, _c_int, _c_int, _c_void_p],
     "ka_pair_embed": [_c_void_p, _c_int, _c_void_p, _c_void_p, _c_int, _c_int, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p,
                       _c_int, _c_long, _c_long, _c_void_p, _c_int, _c_int, _c_int, _c_void_p],
@@ -56,6 +56,17 @@ _SIGNATURES = {
     "ka_matrix_memory": [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_long, _c_int, _c_void_p, _c_void_p, _c_int, _c_void_p,
                          _c_void_p, _c_void_p, _c_void_p, _c_long, _c_int, _c_int, _c_int, _c_int, _c_float, _c_float, _c_float,
                          _c_int, _c_void_p],
+    "ka_token_shift": [_c_void_p, _c_void_p, _c_long, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int,
+                       _c_int, _c_void_p],
+    "ka_decayed_memory": [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_long, _c_int, _c_void_p, _c_void_p, _c_void_p, _c_void_p,
+                          _c_long, _c_void_p, _c_int, _c_void_p, _c_void_p, _c_void_p, _c_long, _c_int, _c_int, _c_int, _c_float,
+                          _c_void_p],
+    "ka_route": [_c_void_p, _c_long, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_void_p, _c_void_p, _c_void_p],
+    "ka_experts_linear": [_c_void_p, _c_long, _c_int, _c_void_p, _c_int, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void_p,
+                          _c_long, _c_int, _c_void_p],
+    "ka_experts_combine": [_c_void_p, _c_void_p, _c_long, _c_int, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_void_p, _c_void_p,
+                           _c_long, _c_void_p, _c_int, _c_int, _c_void_p],
+    "ka_experts_sort": [_c_void_p, _c_int, _c_int, _c_int, _c_int, _c_void_p, _c_void_p, _c_void_p],
     "ka_add_table_rows": [_c_void_p, _c_int, _c_int, _c_void_p, _c_void_p, _c_int, _c_int, _c_void_p],
     "ka_cast_columns": [_c_void_p, _c_void_p, _c_int, _c_long, _c_int, _c_int, _c_void_p],
     "ka_add_scaled": [_c_void_p, _c_void_p, _c_float, _c_long, _c_void_p],
@@ -365,7 +376,8 @@ def qkv_prepare(qkv: torch.Tensor, positions: Optional[torch.Tensor], slots: Opt
                 v_cache: Optional[torch.Tensor], n_heads: int, n_kv_heads: int, head_dim: int, value_dim: int, page_size: int,
                 norm_scope: Optional[str] = None, q_gain: Optional[torch.Tensor] = None, k_gain: Optional[torch.Tensor] = None,
                 eps: float = 0.0, freqs: Optional[torch.Tensor] = None, pairing: str = "halves", q_growth=None,
-                blend: Optional[str] = None, v_other: Optional[torch.Tensor] = None, blend_weight: Optional[torch.Tensor] = None) -> None:
+                blend: Optional[str] = None, v_other: Optional[torch.Tensor] = None, blend_weight: Optional[torch.Tensor] = None,
+                values_from_keys: bool = False) -> None:
     """Queries, keys and values of a step made ready for attention in one pass over ``qkv`` ``[n, H hd | Hkv hd | Hkv hdv]``
     (rows may lie in a wider buffer): the norm of queries and keys (``norm_scope`` ``"head"``: every head by its own root mean
     square, gains ``[hd]``; ``"projection"``: all queries of a token by one, all keys by one, gains ``[H hd]`` and ``[Hkv hd]``),
@@ -373,13 +385,16 @@ def qkv_prepare(qkv: torch.Tensor, positions: Optional[torch.Tensor], slots: Opt
     in ``rope_cache``), then queries times ``1 + coef * ln(floor((place + 1) / every) + 1)`` for ``q_growth = (coef, every)``;
     values copied to ``v_other`` (``blend`` ``"source"``) or replaced by ``(1 - w) v + w v_other`` (``"blend"``, ``w`` the fp32
     scalar tensor ``blend_weight``); queries back in place, keys and values into the paged cache at ``slots`` (the rows keep
-    keys and values as they were projected)."""
+    keys and values as they were projected). ``values_from_keys``: the rows are ``[n, H hd | Hkv hd]`` and the values are the
+    keys as projected (``value_dim`` = ``head_dim``). ``n_kv_heads`` 0: rows of queries alone, nothing is cached."""
     _need(pairing in ROTARY_PAIRINGS, f"qkv_prepare: pairing {pairing!r} is not one of {sorted(ROTARY_PAIRINGS)}")
     _need(norm_scope in QK_NORM_SCOPES and blend in VALUE_BLENDS, "qkv_prepare: unknown norm scope or blend")
     _dev(qkv, positions, slots, k_cache, v_cache, q_gain, k_gain, freqs, v_other, blend_weight)
     n = qkv.shape[0]
-    total = (n_heads + n_kv_heads) * head_dim + n_kv_heads * value_dim
+    total = (n_heads + n_kv_heads) * head_dim + (0 if values_from_keys else n_kv_heads * value_dim)
     _need(qkv.dim() == 2 and qkv.stride(1) == 1 and qkv.shape[1] == total, "qkv_prepare: qkv must be [n, H hd + Hkv hd + Hkv hdv]")
+    _need(not values_from_keys or (value_dim == head_dim and blend is None), "qkv_prepare: values that are the keys have their size")
+    _need(n_kv_heads > 0 or slots is None, "qkv_prepare: rows of queries alone cache nothing")
     for t in (positions, slots):
         _need(t is None or (t.dtype == torch.int32 and t.numel() == n and t.is_contiguous()), "qkv_prepare: per-token int32 [n] expected")
     if slots is not None:
@@ -404,7 +419,8 @@ def qkv_prepare(qkv: torch.Tensor, positions: Optional[torch.Tensor], slots: Opt
                                 _ptr(k_cache), _ptr(v_cache), n, n_heads, n_kv_heads, head_dim, value_dim, page_size,
                                 QK_NORM_SCOPES[norm_scope], _ptr(q_gain), _ptr(k_gain), float(eps), _ptr(freqs), rot,
                                 ROTARY_PAIRINGS[pairing], coef, every, VALUE_BLENDS[blend], _ptr(v_other),
-                                (v_other.stride(0) if n > 1 else n_kv_heads * value_dim) if v_other is not None else 0, _ptr(blend_weight), stream_ptr()))
+                                (v_other.stride(0) if n > 1 else n_kv_heads * value_dim) if v_other is not None else 0, _ptr(blend_weight),
+                                int(bool(values_from_keys)), stream_ptr()))
 
 
 def gated_pairs(x: torch.Tensor, out: torch.Tensor, act: int) -> None:
@@ -638,6 +654,126 @@ def matrix_memory(projected: torch.Tensor, offsets, pre: torch.Tensor, state: to
                                   float(q_scale), float(cap), float(eps), int(bool(single_tokens)), stream_ptr()))
 
 
+def token_shift(x: torch.Tensor, kept: torch.Tensor, mu: torch.Tensor, token_row: torch.Tensor, cu_q: torch.Tensor,
+                row_slot: torch.Tensor, out: torch.Tensor) -> None:
+    """``out[s, t] = x[t] + (x'[t] - x[t]) * mu[s]`` with ``x'[t]`` the stream's row of the token before ``t`` in its sequence: row
+    ``t - 1`` of the step or, for the first token of a row's portion, ``kept[row_slot[row]]`` (zeros where the row has no
+    request). ``x`` fp32 ``[n, dim]``, ``kept`` an fp32 view ``[slots, dim]`` with a row stride of its own, ``mu`` fp32
+    ``[mixes, dim]``, ``out`` ``[mixes, n, dim]``."""
+    _dev(x, kept, mu, token_row, cu_q, row_slot, out)
+    n, dim = x.shape
+    mixes = mu.shape[0]
+    _need(x.dtype == torch.float32 and x.is_contiguous(), "token_shift: x must be contiguous fp32 [n, dim]")
+    _need(mu.dtype == torch.float32 and mu.is_contiguous() and tuple(mu.shape) == (mixes, dim), "token_shift: mu fp32 [mixes, dim]")
+    _need(kept.dtype == torch.float32 and kept.dim() == 2 and kept.shape[1] == dim and kept.stride(1) == 1, "token_shift: kept fp32 [slots, dim]")
+    _need(out.is_contiguous() and tuple(out.shape) == (mixes, n, dim), "token_shift: out must be contiguous [mixes, n, dim]")
+    _need(token_row.dtype == torch.int32 and token_row.numel() == n and cu_q.dtype == torch.int32 and row_slot.dtype == torch.int32
+          and cu_q.numel() == row_slot.numel() + 1, "token_shift: token_row int32 [n], cu_q int32 [rows + 1], row_slot int32 [rows]")
+    _check(lib().ka_token_shift(x.data_ptr(), kept.data_ptr(), kept.stride(0), mu.data_ptr(), token_row.data_ptr(), cu_q.data_ptr(),
+                                row_slot.data_ptr(), out.data_ptr(), code_of(out.dtype), n, dim, mixes, stream_ptr()))
+
+
+def decayed_memory_supported(head_dim: int) -> bool:
+    return bool(lib().ka_decayed_memory_supported(int(head_dim)))
+
+
+def decayed_memory(r: torch.Tensor, k: torch.Tensor, v: torch.Tensor, gate: torch.Tensor, pre: torch.Tensor, u: torch.Tensor,
+                   gain: torch.Tensor, state: torch.Tensor, x: Optional[torch.Tensor], cu_q: torch.Tensor, row_slot: torch.Tensor,
+                   out: torch.Tensor, n_heads: int, head_dim: int, eps: float) -> None:
+    """A decaying matrix memory over the packed tokens of a step. Per head a state ``S`` ``[d, d]``; for every token of a row, in
+    order: ``o_j = sum_i r_i (S_ij + u_i k_i v_j)``, then ``S_ij <- exp(-exp(pre_i)) S_ij + k_i v_j``; ``o`` divided by its root mean
+    square over the head (``eps``), times ``gain``, times ``gate``. ``r, k, v, gate``: ``[n, H d]`` views of one type with one
+    row stride; ``pre`` fp32 ``[n, H d]``; ``u``, ``gain`` fp32 ``[H d]``; ``state`` fp32 ``[slots + 1, H d d + dim]``, a row per
+    request slot: the matrices, then the stream's last row (``x`` fp32 ``[n, dim]``, kept for the next step's token shift;
+    ``None``: the rows hold the matrices alone). A row of the step without a request writes zeros and touches no state."""
+    _dev(r, k, v, gate, pre, u, gain, state, x, cu_q, row_slot, out)
+    n = r.shape[0]
+    width = n_heads * head_dim
+    for t in (r, k, v, gate):
+        _need(t.dtype == r.dtype and t.dim() == 2 and tuple(t.shape) == (n, width) and t.stride(1) == 1 and (n <= 1 or t.stride(0) == r.stride(0)),
+              "decayed_memory: r, k, v and gate must be [n, H d] of one type and row stride")
+    _need(pre.dtype == torch.float32 and pre.is_contiguous() and tuple(pre.shape) == (n, width), "decayed_memory: pre fp32 [n, H d]")
+    for t in (u, gain):
+        _need(t.dtype == torch.float32 and t.is_contiguous() and t.numel() == width, "decayed_memory: u and gain fp32 [H d]")
+    dim = 0 if x is None else x.shape[1]
+    _need(x is None or (x.dtype == torch.float32 and x.is_contiguous() and x.shape[0] == n), "decayed_memory: x fp32 [n, dim]")
+    _need(state.dtype == torch.float32 and state.is_contiguous() and state.dim() == 2 and state.shape[1] == width * head_dim + dim,
+          "decayed_memory: state fp32 [slots, H d d + dim]")
+    n_rows = row_slot.numel()
+    _need(cu_q.dtype == torch.int32 and cu_q.numel() == n_rows + 1 and row_slot.dtype == torch.int32, "decayed_memory: cu_q int32 [rows + 1]")
+    _need(out.dtype == r.dtype and out.dim() == 2 and out.stride(1) == 1 and tuple(out.shape) == (n, width), "decayed_memory: out [n, H d]")
+    _check(lib().ka_decayed_memory(r.data_ptr(), k.data_ptr(), v.data_ptr(), gate.data_ptr(), r.stride(0) if n > 1 else width,
+                                   code_of(r.dtype), pre.data_ptr(), u.data_ptr(), gain.data_ptr(), state.data_ptr(), state.stride(0),
+                                   _ptr(x), dim, cu_q.data_ptr(), row_slot.data_ptr(), out.data_ptr(),
+                                   out.stride(0) if n > 1 else width, n_rows, n_heads, head_dim, float(eps), stream_ptr()))
+
+
+def route(logits: torch.Tensor, n_outputs: int, correction: Optional[torch.Tensor], top: int, n_groups: int, keep_groups: int,
+          scale: float, chosen: torch.Tensor, weights: torch.Tensor) -> None:
+    """A router's choice per token from fp32 ``logits`` ``[n, >= n_outputs]``: scores = softmax over the first ``n_outputs``
+    columns; the choice goes by scores + ``correction`` among the outputs of the ``keep_groups`` best of ``n_groups`` equal
+    groups of neighbours (0 groups: among all); ``chosen`` int32 ``[n, top]``, ``weights`` fp32 ``[n, top]`` = the chosen scores
+    over their sum (+ 1e-20), times ``scale``."""
+    _dev(logits, correction, chosen, weights)
+    n = logits.shape[0]
+    _need(logits.dtype == torch.float32 and logits.dim() == 2 and logits.stride(1) == 1 and logits.shape[1] >= n_outputs, "route: logits fp32 [n, >= outputs]")
+    _need(correction is None or (correction.dtype == torch.float32 and correction.is_contiguous() and correction.numel() == n_outputs),
+          "route: correction fp32 [outputs]")
+    _need(chosen.dtype == torch.int32 and chosen.is_contiguous() and tuple(chosen.shape) == (n, top) and weights.dtype == torch.float32
+          and weights.is_contiguous() and tuple(weights.shape) == (n, top), "route: chosen int32 and weights fp32 [n, top]")
+    _check(lib().ka_route(logits.data_ptr(), logits.stride(0) if n > 1 else logits.shape[1], _ptr(correction), n, int(n_outputs), int(top),
+                          int(n_groups), int(keep_groups), float(scale), chosen.data_ptr(), weights.data_ptr(), stream_ptr()))
+
+
+def experts_linear(a: torch.Tensor, per_token: int, weights: torch.Tensor, chosen: torch.Tensor, out: torch.Tensor, act: int = 0) -> None:
+    """``out[p] = act(a[p // per_token] @ weights[chosen[p]].T)`` for every pair ``p`` whose choice is an expert with weights
+    (``chosen[p] < E``; other rows of ``out`` are left alone). ``weights`` ``[E, N, K]``; ``act`` may carry the gated flag (rows of an
+    expert in pairs). ``out`` of the operands' type or fp32."""
+    _dev(a, weights, chosen, out)
+    n_pairs = chosen.numel()
+    E, N, K = weights.shape
+    n_out = N // 2 if act & 0x100 else N
+    _need(a.dtype == weights.dtype and a.dim() == 2 and a.stride(1) == 1 and a.shape[1] == K and a.shape[0] * per_token >= n_pairs,
+          "experts_linear: a must be [>= pairs / per_token, K] of the weights' type")
+    _need(weights.is_contiguous() and chosen.dtype == torch.int32 and chosen.is_contiguous(), "experts_linear: weights [E, N, K], chosen int32")
+    _need(out.dim() == 2 and out.stride(1) == 1 and tuple(out.shape) == (n_pairs, n_out) and out.dtype in (a.dtype, torch.float32),
+          "experts_linear: out must be [pairs, outputs]")
+    _check(lib().ka_experts_linear(a.data_ptr(), a.stride(0) if a.shape[0] > 1 else K, int(per_token), weights.data_ptr(), code_of(a.dtype),
+                                   chosen.data_ptr(), n_pairs, E, N, K, int(act), out.data_ptr(), out.stride(0) if n_pairs > 1 else n_out,
+                                   int(out.dtype == torch.float32 and a.dtype != torch.float32), stream_ptr()))
+
+
+def experts_combine(y: torch.Tensor, h: torch.Tensor, chosen: torch.Tensor, weights: torch.Tensor, n_experts: int,
+                    shared: Optional[torch.Tensor], shared_gate: Optional[torch.Tensor], out: torch.Tensor, accumulate: bool) -> None:
+    """``out[t] (+)= sum_k weights[t, k] * (y[t * top + k] if chosen[t, k] < n_experts else h[t]) + sigmoid(shared_gate[t]) * shared[t]``.
+    ``y`` fp32 ``[n top, dim]``, ``h`` ``[n, dim]``, ``shared`` fp32 ``[n, dim]`` or ``None``, ``shared_gate`` an fp32 column ``[n]``
+    (a view with a stride) or ``None`` (weight 1), ``out`` fp32 ``[n, dim]``."""
+    _dev(y, h, chosen, weights, shared, shared_gate, out)
+    n, dim = out.shape
+    top = chosen.shape[1]
+    _need(y.dtype == torch.float32 and y.is_contiguous() and tuple(y.shape) == (n * top, dim), "experts_combine: y fp32 [n top, dim]")
+    _need(h.dim() == 2 and tuple(h.shape) == (n, dim) and h.stride(1) == 1, "experts_combine: h [n, dim]")
+    _need(out.dtype == torch.float32 and out.is_contiguous(), "experts_combine: out contiguous fp32")
+    _need(shared is None or (shared.dtype == torch.float32 and shared.is_contiguous() and tuple(shared.shape) == (n, dim)), "experts_combine: shared fp32 [n, dim]")
+    _need(shared_gate is None or (shared_gate.dtype == torch.float32 and shared_gate.dim() == 1 and shared_gate.numel() == n), "experts_combine: the gate is an fp32 column")
+    _check(lib().ka_experts_combine(y.data_ptr(), h.data_ptr(), h.stride(0) if n > 1 else dim, code_of(h.dtype), chosen.data_ptr(),
+                                    weights.data_ptr(), n, top, int(n_experts), _ptr(shared), _ptr(shared_gate),
+                                    (shared_gate.stride(0) if n > 1 else 1) if shared_gate is not None else 0, out.data_ptr(), dim,
+                                    int(bool(accumulate)), stream_ptr()))
+
+
+def experts_sort(chosen: torch.Tensor, n_experts: int, tile: int, sorted_pairs: torch.Tensor, tile_expert: torch.Tensor) -> None:
+    """The pairs listed by expert in runs that start on multiples of ``tile`` rows: ``sorted_pairs`` int32 ``[capacity]`` (-1: an
+    unused row), ``tile_expert`` int32 ``[capacity / tile]`` (-1: a tile behind the last run)."""
+    _dev(chosen, sorted_pairs, tile_expert)
+    capacity = sorted_pairs.numel()
+    _need(chosen.dtype == torch.int32 and chosen.is_contiguous() and sorted_pairs.dtype == torch.int32 and sorted_pairs.is_contiguous()
+          and tile_expert.dtype == torch.int32 and tile_expert.is_contiguous() and tile_expert.numel() * tile == capacity,
+          "experts_sort: int32 lists, capacity a multiple of the tile")
+    _check(lib().ka_experts_sort(chosen.data_ptr(), chosen.numel(), int(n_experts), int(tile), capacity, sorted_pairs.data_ptr(),
+                                 tile_expert.data_ptr(), stream_ptr()))
+
+
 def rope_cache(qkv: torch.Tensor, positions: torch.Tensor, slots: Optional[torch.Tensor],
                table: Optional[torch.Tensor], k_cache: Optional[torch.Tensor], v_cache: Optional[torch.Tensor],
                n_heads: int, n_kv_heads: int, head_dim: int, page_size: int, pairing: str = "halves") -> None:
@@ -696,8 +832,11 @@ def attention_generic(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Ten
                       slopes: Optional[torch.Tensor] = None, sink: Optional[float] = None,
                       bias_table: Optional[torch.Tensor] = None, gate: Optional[torch.Tensor] = None,
                       sinks: Optional[torch.Tensor] = None, keep_first: int = 0, maps: int = 1,
-                      values_in_keys: bool = False) -> None:
+                      values_in_keys: bool = False, softcap: Optional[float] = None, gate_per_head: bool = False) -> None:
     """Paged attention of ``n`` packed tokens; ``q`` may be a strided view into a qkv buffer.
+
+    ``softcap``: the scaled score passes through ``softcap * tanh(score / softcap)``. ``gate_per_head``: ``gate`` is
+    ``[n, H]``, one number per head.
 
     ``sinks`` (fp32 ``[H]``): a score per head for the valueless term instead of the one number ``sink``. ``keep_first``: a
     query also sees the first ``keep_first`` keys of its row where its window (``kv_lo``) has passed them. ``maps`` > 1:
@@ -743,8 +882,10 @@ def attention_generic(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Ten
               and bias_table.is_contiguous(), "attention: the distance table must be contiguous fp32 [H, T]")
         _need(positions is not None and positions.dtype == torch.int32 and positions.numel() == n and positions.is_contiguous(),
               "attention: a distance table needs the queries' positions, int32 [n]")
+    gate_cols = n_heads if gate_per_head else n_heads * value_dim
     _need(gate is None or (gate.is_cuda and gate.dtype == q.dtype and gate.dim() == 2 and gate.stride(1) == 1
-                           and tuple(gate.shape) == (n, n_heads * value_dim)), "attention: the gate must be [n, H hdv] of the q type")
+                           and tuple(gate.shape) == (n, gate_cols)), "attention: the gate must be [n, H hdv] (or [n, H]) of the q type")
+    _need(softcap is None or softcap > 0, "attention: a cap on the scores must be positive")
     _need(block_table.dtype == torch.int32 and block_table.dim() == 2 and block_table.is_contiguous(),
           "attention: block table must be contiguous int32 [rows, pages]")
     for t in (token_row, kv_hi) + ((kv_lo,) if kv_lo is not None else ()):
@@ -756,9 +897,10 @@ def attention_generic(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Ten
                                       value_dim, _ptr(positions) if (slopes is not None or bias_table is not None) else None,
                                       _ptr(slopes), int(sink is not None or sinks is not None), float(sink or 0.0), _ptr(bias_table),
                                       int(bias_table.shape[1]) if bias_table is not None else 0, _ptr(gate),
-                                      (gate.stride(0) if n > 1 else n_heads * value_dim) if gate is not None else 0,
+                                      (gate.stride(0) if n > 1 else gate_cols) if gate is not None else 0,
                                       _ptr(sinks), int(keep_first), maps, int(bool(values_in_keys)),
-                                      int(out.dtype == torch.float32 and q.dtype != torch.float32), stream_ptr()))
+                                      int(out.dtype == torch.float32 and q.dtype != torch.float32), float(softcap or 0.0),
+                                      int(bool(gate_per_head)), stream_ptr()))
 
 
 def _pending_args(who: str, rows: int, pending, pending_at):

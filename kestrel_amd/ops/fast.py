@@ -58,7 +58,7 @@ _SIGNATURES = {
     "ka_attention_biased_bf16": [_c_void_p, _c_long, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_void_p, _c_void_p, _c_int,
                                  _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_long, _c_float,
                                  _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_void_p, _c_int, _c_void_p, _c_long,
-                                 _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void_p, _c_void_p],
+                                 _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void_p, _c_float, _c_int, _c_void_p],
     "ka_heads_linear_bf16": [_c_void_p, _c_long, _c_int, _c_void_p, _c_void_p, _c_long, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void_p,
                              _c_long, _c_void_p],
     "ka_heads_linear_supported": [_c_long, _c_int, _c_long, _c_int, _c_int, _c_int],
@@ -624,7 +624,8 @@ def biased_query_block(head_dim: int, value_dim: int) -> Optional[int]:
 
 def attention_biased_bf16(q, k_cache, v_cache, block_table, token_row, kv_lo, kv_hi, out, scale, n_heads, n_kv_heads,
                           head_dim, value_dim, positions, slopes, sink, batch, bias_table=None, gate=None, sinks=None,
-                          keep_first: int = 0, maps: int = 1, values_in_keys: bool = False) -> bool:
+                          keep_first: int = 0, maps: int = 1, values_in_keys: bool = False, softcap: Optional[float] = None,
+                          gate_per_head: bool = False) -> bool:
     """Attention with the further terms of ``ops.core.attention_generic`` (values of ``value_dim`` channels, ``slopes``
     times the distance taken off the scores, a ``sink`` in the softmax's denominator or one per head in ``sinks``, kept
     first keys before the window, several maps per head over shared values, values that are the first channels of the
@@ -650,9 +651,12 @@ def attention_biased_bf16(q, k_cache, v_cache, block_table, token_row, kv_lo, kv
         raise KernelError("attention: sink scores must be fp32 [H]")
     if slopes is not None and (slopes.dtype != torch.float32 or slopes.numel() != n_heads or positions is None):
         raise KernelError("attention: slopes must be fp32 [H] and come with the queries' positions")
+    gate_cols = n_heads if gate_per_head else n_heads * value_dim
     if gate is not None and (gate.dtype != torch.bfloat16 or gate.dim() != 2 or gate.stride(1) != 1
-                             or tuple(gate.shape) != (n, n_heads * value_dim)):
-        raise KernelError("attention: the output gate must be bf16 [n, H hdv]")
+                             or tuple(gate.shape) != (n, gate_cols)):
+        raise KernelError("attention: the output gate must be bf16 [n, H hdv] (or [n, H])")
+    if softcap is not None and not softcap > 0:
+        raise KernelError("attention: a cap on the scores must be positive")
     if bias_table is not None and (bias_table.dtype != torch.float32 or bias_table.dim() != 2 or bias_table.shape[0] != n_heads
                                    or not bias_table.is_contiguous() or positions is None):
         raise KernelError("attention: the distance table must be contiguous fp32 [H, T] and come with the queries' positions")
@@ -690,8 +694,8 @@ def attention_biased_bf16(q, k_cache, v_cache, block_table, token_row, kv_lo, kv
         _ptr(positions), _ptr(slopes), out.data_ptr(), out.stride(0), float(scale), n, n_heads, n_kv_heads, head_dim,
         value_dim, page_size, waves, int(sink is not None or sinks is not None), float(sink or 0.0), _ptr(bias_table),
         int(bias_table.shape[1]) if bias_table is not None else 0, _ptr(gate),
-        (gate.stride(0) if n > 1 else n_heads * value_dim) if gate is not None else 0, _ptr(sinks), int(keep_first), int(maps),
-        int(bool(values_in_keys)), int(out_f32), n_splits, _ptr(partial), stream_ptr()))
+        (gate.stride(0) if n > 1 else gate_cols) if gate is not None else 0, _ptr(sinks), int(keep_first), int(maps),
+        int(bool(values_in_keys)), int(out_f32), n_splits, _ptr(partial), float(softcap or 0.0), int(bool(gate_per_head)), stream_ptr()))
     return True
 
 
@@ -774,3 +778,9 @@ def matrix_memory_chunks_bf16(projected, offsets, pre, state, cu_q, row_slot, ga
                                                out.stride(0) if n > 1 else n_heads * value_dim, int(row_slot.numel()), n_heads,
                                                head_dim, value_dim, float(q_scale), float(cap), float(eps), _ptr(scratch), n, stream_ptr()))
     return True
+
+
+def experts_feed_forward_bf16(h, pairs, down, chosen, hidden, y, act, workspace) -> bool:
+    """Both linears of the chosen experts for all pairs of a step on the matrix cores, an expert's pairs together. False: not
+    covered, nothing was run."""
+    return False

@@ -10,9 +10,9 @@ from . import core
 
 # The codes of ``KaAct`` in csrc/ka_common.h, which is where a further activation is added (every
 # linear kernel applies them through the same two functions there).
-ACT_NONE, ACT_GELU_TANH, ACT_RELU, ACT_SILU, ACT_RELU_SQUARED = 0, 1, 2, 3, 4
+ACT_NONE, ACT_GELU_TANH, ACT_RELU, ACT_SILU, ACT_RELU_SQUARED, ACT_TANH = 0, 1, 2, 3, 4, 5
 _ACTIVATIONS = {None: ACT_NONE, "none": ACT_NONE, "gelu_tanh": ACT_GELU_TANH, "relu": ACT_RELU, "silu": ACT_SILU,
-                "relu_squared": ACT_RELU_SQUARED}
+                "relu_squared": ACT_RELU_SQUARED, "tanh": ACT_TANH}
 
 # Added to an activation's code: the linear is gated (``KA_ACT_GATED`` in csrc/ka_common.h): weight rows
 # 2j and 2j + 1 are the gate's and the value's of output j, and ``out[:, j] = act(gate sum) * value sum``.

@@ -1,6 +1,6 @@
 """Parts a model is put together from; importing the package registers the built-in kinds."""
 
-from . import (attention, branches, differential_attention, junction, latent_attention, learned_position, matrix_memory, mlp, norm,
+from . import (attention, branches, decayed_memory, differential_attention, experts, junction, latent_attention, learned_position, matrix_memory, mlp, norm,
                pair_embedding, rotary)  # noqa: F401  (registration)
 from .base import (FeedForward, Junction, LayerCache, Mixer, Norm, Part, PositionEncoding, Rotation, SideLinear, build_part, known_kinds,
                    register_feed_forward, register_junction, register_mixer, register_norm, register_position)

@@ -48,6 +48,12 @@ class PagedAttention(Mixer):
     of a further projection of the input before the output projection (``output_gate``, tensor ``gate.weight``, which
     rides in the launch of the q|k|v projection). ``chunk`` is a mask like ``window``: it only changes which keys a
     token reads (``kv_lo``) and which pages go back.
+
+    And four more, again by their fields: values that are the keys as projected (``values_from_keys``: no value
+    projection, the prepare kernel writes the unnormalised, unrotated keys into the value pages); scores capped by
+    ``softcap * tanh(score / softcap)``; a learned sink score per head (``head_sinks``, tensor ``sinks``); a gate of one
+    number per head (``gate_per_head``); and a layer without keys and values of its own (``shares_kv``: it projects
+    queries, and the gate, alone, and its schedule entry reads another entry's cache).
     """
 
     replays_every_step = True
@@ -59,11 +65,19 @@ class PagedAttention(Mixer):
         self.position = build_part("position", spec.position)
         self.scale = float(spec.scale) if spec.scale is not None else float(spec.head_dim) ** -0.5
         self.value_dim = int(spec.head_dim if getattr(spec, "value_dim", None) is None else spec.value_dim)
+        self.shares_kv = bool(getattr(spec, "shares_kv", False))
+        self.values_from_keys = bool(getattr(spec, "values_from_keys", False))
+        if self.values_from_keys and self.value_dim != spec.head_dim:
+            raise ValueError("values that are the keys have the keys' size")
         self.q_dim = spec.n_heads * spec.head_dim
-        self.kv_dim = spec.n_kv_heads * spec.head_dim
-        self.v_dim = spec.n_kv_heads * self.value_dim
+        self.kv_dim = 0 if self.shares_kv else spec.n_kv_heads * spec.head_dim
+        self.v_dim = 0 if (self.shares_kv or self.values_from_keys) else spec.n_kv_heads * self.value_dim
         self.qkv_dim = self.q_dim + self.kv_dim + self.v_dim
         self.out_dim = spec.n_heads * self.value_dim
+        self.softcap = getattr(spec, "softcap", None)
+        self.head_sinks = bool(getattr(spec, "head_sinks", False))
+        self.gate_per_head = bool(getattr(spec, "gate_per_head", False))
+        self._sinks: Optional[torch.Tensor] = None
         self.unit_norm_eps = getattr(spec, "qk_unit_norm_eps", None)
         self.sink = getattr(spec, "sink", None)
         self.distance = getattr(spec, "distance_slopes", None)
@@ -78,11 +92,18 @@ class PagedAttention(Mixer):
         if self.blend is not None and self.blend.role not in ("source", "blend"):
             raise ValueError(f"a value blend has the role 'source' or 'blend', got {self.blend.role!r}")
         self.extended = self.value_dim != spec.head_dim or self.unit_norm_eps is not None or self.sink is not None \
-            or self.distance is not None or self.buckets is not None
+            or self.distance is not None or self.buckets is not None or self.softcap is not None or self.head_sinks \
+            or (self.gated and self.gate_per_head)
         # the forms that ``ops.core.qkv_prepare`` makes ready (a rotation by frequencies, found when the weights are bound, too)
         self.prepared = self.qk_norm is not None or self.growth is not None or self.buckets is not None \
-            or self.blend is not None or self.gated
-        self.in_dim = self.qkv_dim + (self.out_dim if self.gated else 0)
+            or self.blend is not None or self.gated or self.shares_kv or self.values_from_keys or self.softcap is not None \
+            or self.head_sinks
+        if (self.shares_kv or self.values_from_keys) and (self.unit_norm_eps is not None or self.blend is not None):
+            raise ValueError("a layer without values of its own takes neither unit-norm keys nor blended values")
+        if self.head_sinks and self.sink is not None:
+            raise ValueError("a sink is one number (sink) or one per head (head_sinks), not both")
+        self.gate_dim = (spec.n_heads if self.gate_per_head else self.out_dim) if self.gated else 0
+        self.in_dim = self.qkv_dim + self.gate_dim
         self._slopes: Optional[torch.Tensor] = None
         self._bias_table: Optional[torch.Tensor] = None
         self._q_gain = self._k_gain = self._blend_weight = self._freqs = None
@@ -93,16 +114,19 @@ class PagedAttention(Mixer):
 
     def params(self) -> Dict[str, ParamSpec]:
         spec = self.spec
-        pieces = {"q": self.q_dim, "k": self.kv_dim, "v": self.v_dim} if getattr(spec, "split_projections", False) \
-            else {"qkv": self.qkv_dim}
+        pieces = {name: rows for name, rows in (("q", self.q_dim), ("k", self.kv_dim), ("v", self.v_dim)) if rows} \
+            if getattr(spec, "split_projections", False) else {"qkv": self.qkv_dim}
         out = {f"{name}.weight": ParamSpec((rows, spec.dim)) for name, rows in pieces.items()}
         out["proj.weight"] = ParamSpec((spec.dim, self.out_dim))
         if self.gated:
-            out["gate.weight"] = ParamSpec((self.out_dim, spec.dim))
+            out["gate.weight"] = ParamSpec((self.gate_dim, spec.dim))
         if self.qk_norm is not None and self.qk_norm.gain:
             per_head = self.qk_norm.scope == "head"
             out["q_norm.weight"] = ParamSpec((spec.head_dim if per_head else self.q_dim,), "vector", "gain")
-            out["k_norm.weight"] = ParamSpec((spec.head_dim if per_head else self.kv_dim,), "vector", "gain")
+            if not self.shares_kv:
+                out["k_norm.weight"] = ParamSpec((spec.head_dim if per_head else self.kv_dim,), "vector", "gain")
+        if self.head_sinks:
+            out["sinks"] = ParamSpec((spec.n_heads,), "vector", "bias")
         if self.buckets is not None:
             out["rel"] = ParamSpec((-1 if self.buckets.buckets is None else self.buckets.buckets, spec.n_heads), "matrix", "bias")
         if self.blend is not None:
@@ -124,7 +148,7 @@ class PagedAttention(Mixer):
         def fused(what: str) -> torch.Tensor:
             # (rows of q, then k, then v: the order of a fused projection's outputs)
             if split:
-                return torch.cat([tensors[f"{name}.{what}"].to(device) for name in ("q", "k", "v")], dim=0)
+                return torch.cat([tensors[f"{name}.{what}"].to(device) for name in ("q", "k", "v") if f"{name}.{what}" in tensors], dim=0)
             return tensors[f"qkv.{what}"].to(device)
 
         self.qkv_weight = fused("weight").contiguous()
@@ -136,10 +160,13 @@ class PagedAttention(Mixer):
             # the gate's rows behind those of q, k and v: one launch projects all four (the gate has no bias)
             self.qkv_weight = torch.cat([self.qkv_weight, tensors["gate.weight"].to(device)], dim=0).contiguous()
             if self.qkv_bias is not None:
-                self.qkv_bias = torch.cat([self.qkv_bias, torch.zeros(self.out_dim, dtype=torch.float32, device=device)]).contiguous()
+                self.qkv_bias = torch.cat([self.qkv_bias, torch.zeros(self.gate_dim, dtype=torch.float32, device=device)]).contiguous()
         if self.qk_norm is not None and self.qk_norm.gain:
             self._q_gain = tensors["q_norm.weight"].to(device=device, dtype=torch.float32).contiguous()
-            self._k_gain = tensors["k_norm.weight"].to(device=device, dtype=torch.float32).contiguous()
+            if not self.shares_kv:
+                self._k_gain = tensors["k_norm.weight"].to(device=device, dtype=torch.float32).contiguous()
+        if self.head_sinks:
+            self._sinks = tensors["sinks"].to(device=device, dtype=torch.float32).contiguous()
         if self.buckets is not None:
             # rel [buckets, H] -> the bias by distance [H, distances]: the kernels look a distance up, not its bucket
             buckets = self.buckets.sized(tensors["rel"].shape[0])
@@ -164,7 +191,7 @@ class PagedAttention(Mixer):
             if freqs.dtype != torch.float32 or freqs.dim() != 1 or 2 * freqs.numel() > spec.head_dim:
                 raise ValueError(f"a rotation's frequencies must be fp32 [R / 2] with R at most the head size {spec.head_dim}")
             if self.unit_norm_eps is not None or self.sink is not None or self.distance is not None:
-                raise ValueError("attention with unit-norm queries and keys, distance slopes or a sink takes no rotation")
+                raise ValueError("attention with unit-norm queries and keys, distance slopes or a one-number sink takes no rotation")
             self._freqs, self._pairing, self._table = freqs.to(device).contiguous(), rotation.pairing, None
             self.prepared = True
         elif rotation is not None:
@@ -288,12 +315,16 @@ class PagedAttention(Mixer):
             # the source layer's values of this step's tokens: scratch of the step, at a fixed address under graphs
             other = batch.workspace.get("shared." + self.blend.name, (n, self.v_dim), self.dtype)
         norm = self.qk_norm
-        core.qkv_prepare(qkv, batch.positions, slots, cache.k, cache.v, spec.n_heads, spec.n_kv_heads, spec.head_dim,
-                         self.value_dim, group.page_size, norm.scope if norm is not None else None, self._q_gain, self._k_gain,
-                         float(norm.eps) if norm is not None else 0.0, self._freqs, self._pairing,
+        if self.shares_kv and cache.writes:
+            raise RuntimeError("a layer without keys and values of its own must read another layer's cache (ScheduleEntry.reads_cache_of)")
+        core.qkv_prepare(qkv, batch.positions, slots, cache.k, cache.v, spec.n_heads, 0 if self.shares_kv else spec.n_kv_heads,
+                         spec.head_dim, self.value_dim, group.page_size, norm.scope if norm is not None else None, self._q_gain,
+                         self._k_gain, float(norm.eps) if norm is not None else 0.0, self._freqs, self._pairing,
                          (self.growth.coef, self.growth.every) if self.growth is not None else None,
-                         self.blend.role if self.blend is not None else None, other, self._blend_weight)
+                         self.blend.role if self.blend is not None else None, other, self._blend_weight,
+                         values_from_keys=self.values_from_keys)
         gate = projected[:, self.qkv_dim:] if self.gated else None
+        more = dict(sinks=self._sinks, softcap=self.softcap, gate_per_head=self.gate_per_head)
         done = gated = False          # (gated: the attention kernel has applied the output gate in its epilogue)
         if qkv.dtype == torch.bfloat16:
             from ..ops import fast
@@ -301,7 +332,7 @@ class PagedAttention(Mixer):
                 done = gated = fast.attention_biased_bf16(qkv, cache.k, cache.v, group.block_table, batch.token_row, group.kv_lo,
                                                           batch.kv_hi, out, self.scale, spec.n_heads, spec.n_kv_heads, spec.head_dim,
                                                           self.value_dim, batch.positions, None, None, batch,
-                                                          bias_table=self._bias_table, gate=gate)
+                                                          bias_table=self._bias_table, gate=gate, **more)
             else:
                 paged_attention(qkv, cache.k, cache.v, group.block_table, batch.token_row, group.kv_lo, batch.kv_hi, out,
                                 self.scale, spec.n_heads, spec.n_kv_heads, spec.head_dim, batch)
@@ -309,7 +340,7 @@ class PagedAttention(Mixer):
         if not done:
             core.attention_generic(qkv, cache.k, cache.v, group.block_table, batch.token_row, group.kv_lo, batch.kv_hi, out,
                                    self.scale, spec.n_heads, spec.n_kv_heads, spec.head_dim, self.value_dim, batch.positions,
-                                   None, None, bias_table=self._bias_table, gate=gate)
+                                   None, None, bias_table=self._bias_table, gate=gate, **more)
             gated = True
         if self.gated and not gated:
             core.gate_mul(out, gate)

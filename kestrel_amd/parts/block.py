@@ -236,8 +236,52 @@ def _parallel_two_norms(block: "Block", x, batch, cache) -> None:
 _parallel_two_norms.defers = True
 
 
+def _output_norms(block: "Block", x, batch, cache) -> None:
+    """``x += norm(mixer(x)); x += norm2(ff(x))``: the parts read the stream itself (rounded to the activation type, or,
+    for a mixer that says ``reads_stream``, as it is) and the norms stand behind them. Each part writes its output into
+    an fp32 buffer (``mix``; a part without it adds into a cleared buffer through ``forward``), and the norm's kernel adds
+    the normalised rows into the stream (``Norm.add_normed``)."""
+    from ..ops import core
+
+    ws = batch.workspace
+    delta = ws.get("block.delta", tuple(x.shape), torch.float32)
+
+    def rounded():
+        if block.dtype == torch.float32:
+            return x
+        h = ws.get("block.h", tuple(x.shape), block.dtype)
+        core.cast_columns(x, h)
+        return h
+
+    def add(norm) -> None:
+        if callable(getattr(norm, "add_normed", None)):
+            norm.add_normed(delta, x)
+        else:
+            normed = ws.get("block.normed", tuple(x.shape), torch.float32)
+            norm.forward(delta, normed)
+            core.add_scaled(x, normed, 1.0)
+
+    mixer = block.mixer
+    source = x if getattr(mixer, "reads_stream", False) else rounded()
+    if callable(getattr(mixer, "mix", None)):
+        mixer.mix(source, batch, cache, delta, False)
+    else:
+        delta.zero_()
+        mixer.forward(source, batch, cache, delta)
+    add(block.norm)
+    ff = block.feed_forward
+    if ff is not None:
+        h = rounded()
+        if callable(getattr(ff, "mix", None)):
+            ff.mix(h, batch, delta, False)
+        else:
+            delta.zero_()
+            ff.forward(h, batch, delta)
+        add(block.norm2)
+
+
 ARRANGEMENTS: Dict[str, Callable] = {"parallel": _parallel, "sequential": _sequential,
-                                     "parallel_two_norms": _parallel_two_norms}
+                                     "parallel_two_norms": _parallel_two_norms, "output_norms": _output_norms}
 
 
 def register_arrangement(name: str, fn: Callable) -> None:
@@ -261,7 +305,9 @@ class Block:
         if spec.arrangement == "sequential" and self.norm2 is None and spec.feed_forward is not None:
             raise ValueError("the sequential arrangement needs norm2 for its feed-forward")
         self.mixer = build_part("mixer", spec.mixer)
-        if spec.feed_forward is None and spec.arrangement not in ("parallel_two_norms", "parallel", "sequential"):
+        if spec.arrangement == "output_norms" and self.norm2 is None and spec.feed_forward is not None:
+            raise ValueError("the output_norms arrangement needs norm2 for its feed-forward")
+        if spec.feed_forward is None and spec.arrangement not in ("parallel_two_norms", "parallel", "sequential", "output_norms"):
             raise ValueError(f"the {spec.arrangement} arrangement needs a feed-forward")
         if spec.arrangement == "parallel_two_norms" and spec.feed_forward is not None and self.norm2 is None:
             raise ValueError("the parallel_two_norms arrangement needs norm2 for its feed-forward")

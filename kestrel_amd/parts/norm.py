@@ -44,8 +44,9 @@ class LayerNorm(Norm):
 
 
 class RMSNorm(Norm):
-    """``x / sqrt(mean(x^2) + eps) * weight`` over the last axis: no mean is taken off, no shift is added, the
-    weight is used as stored (not as one plus it). It offers no ``layernorm_operands`` (it is no LayerNorm), but
+    """``x / sqrt(mean(x^2) + eps) * (offset + weight)`` over the last axis: no mean is taken off, no shift is added;
+    ``spec.offset`` is 0 for a weight used as stored and 1 for one stored around zero (added once, in fp32, when the
+    weights are bound). It offers no ``layernorm_operands`` (it is no LayerNorm), but
     ``rms_operands``: the weight-streaming linears of a few rows take it into their launch as they take a LayerNorm."""
 
     replays_every_step = True
@@ -55,13 +56,18 @@ class RMSNorm(Norm):
         self.weight: Optional[torch.Tensor] = None
 
     def params(self) -> Dict[str, ParamSpec]:
-        return {"weight": ParamSpec((self.spec.dim,), "vector", "gain")}
+        around_zero = float(getattr(self.spec, "offset", 0.0)) != 0.0
+        return {"weight": ParamSpec((self.spec.dim,), "vector", "shift" if around_zero else "gain")}
 
     def bind(self, tensors, dtype, device) -> None:
-        self.weight = tensors["weight"].to(device=device, dtype=torch.float32).contiguous()
+        self.weight = (tensors["weight"].to(device=device, dtype=torch.float32) + float(getattr(self.spec, "offset", 0.0))).contiguous()
 
     def forward(self, x, out, rows=None) -> None:
         core.rmsnorm(x, self.weight, self.spec.eps, out, rows)
+
+    def add_normed(self, y, x) -> None:
+        """``x += norm(y)`` for fp32 rows ``y`` into the fp32 stream ``x`` (a norm that stands behind a sublayer)."""
+        core.branches_sum(x, y, self.weight, 1.0, eps=float(self.spec.eps))
 
     def rms_operands(self):
         """``(weight fp32 [dim], eps)`` of ``x / sqrt(mean(x^2) + eps) * weight``."""

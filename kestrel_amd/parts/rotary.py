@@ -46,13 +46,16 @@ class NeoxRotary(PositionEncoding):
 
 def rotary_frequencies(rotary_dim: int, theta: float, scaling=None):
     """``f_i = theta ** (-2 i / rotary_dim)`` for the ``rotary_dim / 2`` pairs, rescaled by wavelength where a
-    ``WavelengthScaling`` is given (long wavelengths divided by its factor, short ones kept, a linear blend between)."""
+    ``WavelengthScaling`` is given (long wavelengths divided by its factor, short ones kept, a linear blend between),
+    or all divided by the factor of a ``LinearScaling``."""
     import math
 
     out = []
     for i in range(rotary_dim // 2):
         f = float(theta) ** (-2.0 * i / rotary_dim)
-        if scaling is not None:
+        if scaling is not None and not hasattr(scaling, "original"):
+            f = f / float(scaling.factor)
+        elif scaling is not None:
             wavelength = 2.0 * math.pi / f
             if wavelength > scaling.original / scaling.low:
                 f = f / scaling.factor
@@ -66,7 +69,7 @@ def rotary_frequencies(rotary_dim: int, theta: float, scaling=None):
 class FrequencyRotary(PositionEncoding):
     """A rotation given by its frequencies alone: the kernels compute the angle ``place * f_i`` and its cosine and sine
     in fp32 themselves, so there is no table and no longest sequence. ``spec.pairing`` says which channels angle ``i``
-    turns (``"halves"`` or ``"interleaved"``), ``spec.scaling`` rescales the frequencies by wavelength."""
+    turns (``"halves"`` or ``"interleaved"``), ``spec.scaling`` rescales the frequencies (by wavelength, or all alike)."""
 
     replays_every_step = True
 

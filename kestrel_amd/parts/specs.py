@@ -32,10 +32,13 @@ class ParamSpec:
 
 @dataclass(frozen=True)
 class NormSpec:
+    """``offset``: what is added to the stored weight before it multiplies (1.0 for a weight stored around zero)."""
+
     kind: str
     dim: int
     eps: float
     bias: bool = True
+    offset: float = 0.0
 
 
 @dataclass(frozen=True)
@@ -51,6 +54,13 @@ class WavelengthScaling:
 
 
 @dataclass(frozen=True)
+class LinearScaling:
+    """Rotary frequencies all divided by ``factor`` (positions stretched evenly)."""
+
+    factor: float
+
+
+@dataclass(frozen=True)
 class PositionSpec:
     """Position encoding applied inside a mixer. ``kind`` ``none`` encodes nothing. ``pairing`` and ``scaling`` are
     read by the kind ``rotary`` (angles computed from frequencies, no table and so no longest sequence)."""
@@ -60,7 +70,7 @@ class PositionSpec:
     theta: float = 0.0
     max_positions: int = 0
     pairing: str = "halves"
-    scaling: Optional[WavelengthScaling] = None
+    scaling: Optional[object] = None       # ``WavelengthScaling`` or ``LinearScaling``
 
 
 @dataclass(frozen=True)
@@ -275,6 +285,18 @@ class AttentionSpec:
     value_blend: Optional[ValueBlend] = None
     # the concatenated heads multiplied by ``sigmoid(gate.weight @ input)`` before the output projection
     output_gate: bool = False
+    # the gate is one number per head (``gate.weight`` ``[n_heads, dim]``) instead of one per channel
+    gate_per_head: bool = False
+    # the values are the keys as projected, before any norm or rotation: there is no value projection
+    # (``value_dim`` must be the head size)
+    values_from_keys: bool = False
+    # scores pass through ``softcap * tanh(score / softcap)`` after the scale
+    softcap: Optional[float] = None
+    # a learned score per head (tensor ``sinks`` ``[n_heads]``) for the valueless term of the softmax's denominator
+    head_sinks: bool = False
+    # the layer has no keys and values of its own: its schedule entry reads the cache of another (``reads_cache_of``),
+    # and it holds no tensors of key and value projections or of their norm
+    shares_kv: bool = False
 
 
 @dataclass(frozen=True)
@@ -390,6 +412,46 @@ class GatedFeedForwardSpec:
 
 
 @dataclass(frozen=True)
+class RoutedExpertsSpec:
+    """A mixture of gated feed-forwards ``down(act(gate h) * (up h))`` of which every token uses ``top``.
+
+    The router has ``n_experts + n_identity`` outputs; its scores are their softmax (fp32). The choice goes by the scores
+    plus a stored correction (tensor ``correction``), the weights by the scores alone: the chosen scores divided by
+    their sum (+ 1e-20), times ``scale``. ``n_groups`` > 0: the router's outputs form that many equal groups of
+    neighbours, a group counts by its largest choice score, and only outputs of the ``keep_groups`` best groups can be
+    chosen. The last ``n_identity`` outputs are experts without tensors whose output is the input itself.
+    ``shared_hidden``: a further expert of that hidden size that every token uses, times ``sigmoid(shared.sg h)`` (one
+    number per token) if ``shared_gate``."""
+
+    kind: str
+    dim: int
+    n_experts: int
+    hidden_dim: int
+    top: int
+    scale: float = 1.0
+    n_identity: int = 0
+    n_groups: int = 0
+    keep_groups: int = 0
+    activation: str = "silu"
+    shared_hidden: Optional[int] = None
+    shared_gate: bool = True
+
+
+@dataclass(frozen=True)
+class DecayedMemorySpec:
+    """A recurrent mixer in the manner of RWKV's time mixing: per head a state ``S`` ``[head_dim, head_dim]`` that decays
+    channel by channel by a factor computed from the input (``parts/decayed_memory.py``). ``decay_rank``: the size of the
+    low-rank bottleneck of the decay's projection (``None``: as the weights file has it)."""
+
+    kind: str
+    dim: int
+    n_heads: int
+    head_dim: int
+    eps: float                      # of the norm of every head's read-out
+    decay_rank: Optional[int] = None
+
+
+@dataclass(frozen=True)
 class MatrixMemorySpec:
     """A recurrent mixer whose state per head is a matrix ``[head_dim, value_dim]`` with a normaliser and a running
     maximum, written through exponential input and forget gates (``parts/matrix_memory.py``)."""
@@ -424,6 +486,8 @@ class LayerSpec:
     ``sequential`` = ``x += mixer(norm(x)); x += ff(norm2(x))`` (``feed_forward`` and ``norm2`` may be ``None``: a mixer alone);
     ``parallel_two_norms`` = ``x + residual_scale * (mixer(norm(x)) + ff(norm2(x)))``, both norms of the same ``x``
     (``feed_forward`` and ``norm2`` may be ``None`` there: a layer of a mixer alone).
+    ``output_norms`` = ``x += norm(mixer(x)); x += norm2(ff(x))``: the parts read the stream itself and the norms stand
+    behind them (``feed_forward`` and ``norm2`` may be ``None``).
     ``names`` maps ``"<part>.<local tensor name>"`` (parts: ``norm``, ``norm2``, ``mixer``,
     ``feed_forward``) to the tensor's name in the checkpoint.
     """
