@@ -31,7 +31,7 @@ ARCH = "gfx950"
 LIBRARIES: Dict[str, List[str]] = {
     "core": ["ka_error.hip", "elementwise.hip", "gemm_generic.hip", "attention_generic.hip", "mixer_parts.hip", "sequence_parts.hip", "recurrent_parts.hip", "experts.hip",
              "sampling.hip", "peaks.hip"],
-    "fast": ["ka_error.hip", "gemm_bf16.hip", "gemv_bf16.hip", "attention_bf16.hip", "attention_biased_bf16.hip", "heads_linear_bf16.hip", "matrix_memory_bf16.hip", "decode_beside.hip",
+    "fast": ["ka_error.hip", "gemm_bf16.hip", "gemv_bf16.hip", "attention_bf16.hip", "attention_biased_bf16.hip", "heads_linear_bf16.hip", "matrix_memory_bf16.hip", "decode_beside.hip", "experts_bf16.hip",
              "gemm_library.hip"],
 }
 HEADERS = ["ka_common.h", "ka_partials.h", "ka_no_alloc.h", "ka_attention_decode.h", "ka_skinny.h"]

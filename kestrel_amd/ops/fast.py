@@ -62,6 +62,9 @@ _SIGNATURES = {
     "ka_heads_linear_bf16": [_c_void_p, _c_long, _c_int, _c_void_p, _c_void_p, _c_long, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void_p,
                              _c_long, _c_void_p],
     "ka_heads_linear_supported": [_c_long, _c_int, _c_long, _c_int, _c_int, _c_int],
+    "ka_experts_gemm_supported": [_c_long, _c_int, _c_int, _c_long, _c_int, _c_int],
+    "ka_experts_gemm_bf16": [_c_void_p, _c_long, _c_int, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_void_p,
+                             _c_long, _c_int, _c_int, _c_void_p],
     "ka_matrix_memory_chunks_bf16": [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_long, _c_void_p, _c_void_p, _c_void_p, _c_void_p,
                                      _c_void_p, _c_void_p, _c_long, _c_int, _c_int, _c_int, _c_int, _c_float, _c_float, _c_float,
                                      _c_void_p, _c_int, _c_void_p],
@@ -168,6 +171,8 @@ def lib():
             getattr(handle, name).restype = _c_int
         handle.ka_attention_biased_supported.argtypes = [_c_int] * 3
         handle.ka_attention_biased_supported.restype = _c_int
+        handle.ka_experts_gemm_tile.argtypes = []
+        handle.ka_experts_gemm_tile.restype = _c_int
         handle.ka_attention_biased_query_block.argtypes = []
         handle.ka_attention_biased_query_block.restype = _c_int
         handle.ka_attention_decode_beside_supported.argtypes = [_c_int] * 6
@@ -781,6 +786,35 @@ def matrix_memory_chunks_bf16(projected, offsets, pre, state, cu_q, row_slot, ga
 
 
 def experts_feed_forward_bf16(h, pairs, down, chosen, hidden, y, act, workspace) -> bool:
-    """Both linears of the chosen experts for all pairs of a step on the matrix cores, an expert's pairs together. False: not
-    covered, nothing was run."""
-    return False
+    """Both linears of the chosen experts for all pairs of a step on the matrix cores, an expert's pairs together: the pairs
+    are listed by expert (``ops.core.experts_sort``), the gated first linear gathers every pair's token from ``h`` ``[n, dim]`` and
+    leaves the hidden rows in list order, the second writes fp32 ``y`` ``[n top, dim]`` at the pairs' own rows. ``pairs``
+    ``[E, 2 hidden, dim]``, ``down`` ``[E, dim, hidden]``, ``chosen`` int32 ``[n, top]``; ``hidden`` is not used (the list's hidden rows
+    live in the workspace). False: not covered (sizes that are no multiple of 16, alignment), nothing was run."""
+    from . import core
+    n, top = chosen.shape
+    n_experts, n_pair_rows, dim = pairs.shape
+    ff = down.shape[2]
+    handle = lib()
+    if h.dtype != torch.bfloat16 or pairs.dtype != torch.bfloat16 or down.dtype != torch.bfloat16 or y.dtype != torch.float32 \
+            or h.stride(1) != 1 or not pairs.is_contiguous() or not down.is_contiguous() or not y.is_contiguous() \
+            or h.data_ptr() % 16 or pairs.data_ptr() % 16 or down.data_ptr() % 16 or y.data_ptr() % 16:
+        return False
+    lda = h.stride(0) if n > 1 else dim
+    gated = int(act) | ACT_GATED
+    if not handle.ka_experts_gemm_supported(lda, n_pair_rows, dim, ff, gated, 0) or not handle.ka_experts_gemm_supported(ff, dim, ff, dim, 0, 1):
+        return False
+    tile = int(handle.ka_experts_gemm_tile())
+    # (sized by the step's tokens alone: the same for every replay of a captured step)
+    capacity = -(-(n * top + n_experts * (tile - 1)) // tile) * tile
+    if capacity // tile > 65535:
+        return False
+    listed = workspace.get("experts.sorted", (capacity,), torch.int32)
+    tile_expert = workspace.get("experts.tile_expert", (capacity // tile,), torch.int32)
+    rows = workspace.get("experts.hidden_listed", (capacity, ff), torch.bfloat16)
+    core.experts_sort(chosen.view(-1), n_experts, tile, listed, tile_expert)
+    _check(handle.ka_experts_gemm_bf16(h.data_ptr(), lda, top, pairs.data_ptr(), listed.data_ptr(), tile_expert.data_ptr(), capacity // tile,
+                                       n_pair_rows, dim, gated, rows.data_ptr(), ff, 0, 0, stream_ptr()))
+    _check(handle.ka_experts_gemm_bf16(rows.data_ptr(), ff, 0, down.data_ptr(), listed.data_ptr(), tile_expert.data_ptr(), capacity // tile,
+                                       dim, ff, 0, y.data_ptr(), dim, 1, 1, stream_ptr()))
+    return True
