@@ -20,6 +20,7 @@ feed-forward, heads, head size, runs of layers, vocabulary; random weights): a p
 8 and 64 through the same step function, each with its share of the roofline (``--compare-sizes``, ``--compare-model``).
 ``--workload compare-bogivik`` does the same for the Bogivik design (layers of attention with a distance bias and a
 layer of chunked attention beside a matrix memory) at sizes of its own (``BOGIVIK_SIZES``), and
+``--workload compare-bokorax`` for the Bokorax design (two kinds of attention, a decaying matrix memory, routed experts),
 ``--workload compare-letevik`` for the Letevik design (differential attention behind short convolutions and latent
 attention in a looped stretch of layers; ``LETEVIK_SIZES``).
 """
@@ -231,7 +232,7 @@ def design_facts(net):
     plan = net.plan
     embedding = plan.names["embedding"]
     linear = sum(int(__import__("math").prod(p.shape)) for name, p in net.params().items() if p.role == "matrix" and name != embedding)
-    attention, memory = [], []
+    attention, memory, experts = [], [], []
 
     def walk(spec):
         kind = getattr(spec, "kind", None)
@@ -250,13 +251,22 @@ def design_facts(net):
             attention.append((spec.n_heads * (spec.head_dim + spec.rot_dim + spec.value_dim), spec.kv_rank + spec.rot_dim, None, None, 0))
         elif kind == "matrix_memory":
             memory.append((spec.n_heads, spec.head_dim, spec.value_dim))
+        elif kind == "decayed_memory":
+            memory.append((spec.n_heads, spec.head_dim, spec.head_dim))
         elif kind == "branches":
             for branch in spec.branches:
                 walk(branch)
 
     for entry in plan.schedule:
         walk(plan.layers[entry.layer].mixer)
-    return SimpleNamespace(linear=linear, attention=attention, memory=memory, width=plan.dim, vocab=plan.vocab_size)
+        ff = plan.layers[entry.layer].feed_forward
+        if getattr(ff, "kind", None) == "routed_experts":
+            # routed experts: a token multiplies with `top` of them, and a step reads those that its tokens chose; they are
+            # counted apart from the weights that every token uses
+            size = 3 * ff.dim * ff.hidden_dim
+            experts.append((ff.n_experts, ff.top, size))
+            linear -= ff.n_experts * size
+    return SimpleNamespace(linear=linear, attention=attention, memory=memory, experts=experts, width=plan.dim, vocab=plan.vocab_size)
 
 
 def _keys_seen(place: int, window, chunk, keep_first: int = 0) -> int:
@@ -276,6 +286,8 @@ def design_flops(f, tokens: int) -> float:
         total += 2.0 * per_key * sum(_keys_seen(p, window, chunk, kept) for p in range(tokens))
     for h, d, dv in f.memory:
         total += 2.0 * 2.0 * h * d * dv * tokens
+    for _count, top, size in getattr(f, "experts", ()):
+        total += 2.0 * tokens * top * size
     return total
 
 
@@ -287,6 +299,8 @@ def design_decode_bytes(f, batch: int, context: int, size: int) -> float:
         total += size * batch * held * _keys_seen(context, window, chunk, kept)
     for h, d, dv in f.memory:
         total += 2.0 * 4 * batch * h * (d * dv + d + 1)
+    for count, top, expert_size in getattr(f, "experts", ()):
+        total += float(size) * min(count, batch * top) * expert_size          # (at most: rows may choose the same experts)
     return total
 
 
@@ -328,6 +342,58 @@ def letevik_models(size: dict, positions: int):
                           "max_context": positions, "n_heads": md["heads"], "n_kv_heads": md["kv_heads"], "head_dim": md["head"],
                           "rotary_dim": md["head"] // 2, "rope_theta": 10000.0, "prefix_attn": 0, "layer_norm_eps": 1e-5}}
     return {"letevik": (letevik, "letevik"), "moondream2": (moondream, "moondream2")}
+
+
+# Sizes at which Bokorax is measured beside the Moondream decoder: width, heads, kv heads and head size of both kinds of
+# attention, the window of the first kind, heads and head size of the decaying memory, the routed experts (how many, their
+# hidden size, choices per token, identity experts, groups and kept groups) and the shared expert, and the order of layers
+# (2: capped attention with sinks, w: the decaying memory, 1: windowed attention whose values are its keys, s: capped
+# attention that reads the keys and values of the first capped layer). A token multiplies with `top` experts and the shared
+# one: as many feed-forward weights as Moondream's plain feed-forward of one and a half times `ff`.
+BOKORAX_SIZES = {
+    "w2048": dict(width=2048, ff=5632, heads=32, kv_heads=8, head=64, window=1024, memory=(32, 64), rank=64,
+                  experts=dict(n=30, ff=704, top=4, identity=2, groups=(4, 2), shared=2816), order="2w1s"),
+    "w4096": dict(width=4096, ff=7168, heads=32, kv_heads=8, head=128, window=2048, memory=(64, 64), rank=128,
+                  experts=dict(n=62, ff=896, top=6, identity=2, groups=(8, 4), shared=1792), order="w21"),
+}
+
+
+def bokorax_models(size: dict, positions: int):
+    """``{name: (config dict, registry name)}`` of Bokorax and of the Moondream decoder at one size."""
+    h, g, d, w = size["heads"], size["kv_heads"], size["head"], size["width"]
+    e = size["experts"]
+    mlp = {"kind": "moe", "expert": {"ff": e["ff"]}, "shared": {"ff": e["shared"]},
+           "router": {"experts": e["n"], "top": e["top"], "identity": e["identity"], "scale": 2.5,
+                      "groups": {"count": e["groups"][0], "keep": e["groups"][1]}}}
+    first = {"heads": h, "kv_heads": g, "dim": d, "vdim": d, "scale": d ** -0.5, "mask": {"size": size["window"]},
+             "rot": {"base": 10000.0, "dims": d // 2}}
+    second = {"heads": h, "kv_heads": g, "dim": d, "vdim": d, "scale": d ** -0.5, "softcap": 50.0,
+              "rot": {"base": 500000.0, "dims": d, "scaling": {"factor": 8.0}}}
+    memory = {"heads": size["memory"][0], "dim": size["memory"][1], "decay_rank": size["rank"]}
+    layers, source = [], None
+    for i, kind in enumerate(size["order"]):
+        if kind == "w":
+            layers.append({"type": "wkv", "mixer": dict(memory), "mlp": mlp})
+        elif kind == "1":
+            layers.append({"type": "attention", "mixer": dict(first), "mlp": mlp})
+        else:
+            mixer = dict(second)
+            if kind == "s":
+                mixer["kv_from"] = source
+            else:
+                source = i if source is None else source
+            layers.append({"type": "attention_2", "mixer": mixer, "mlp": mlp})
+    bokorax = {"architecture": "Bokorax", "vocab": COMPARE_VOCAB, "width": w, "norm": {"eps": 1e-6}, "max_positions": positions,
+               "embedding": {"scale": 1.0}, "logit_scale": 1.0, "layers": layers}
+    moondream = {"text": {"dim": w, "ff_dim": size["ff"] * 3 // 2, "n_layers": len(size["order"]), "vocab_size": COMPARE_VOCAB,
+                          "max_context": positions, "n_heads": h, "n_kv_heads": g, "head_dim": d, "rotary_dim": d // 2,
+                          "rope_theta": 10000.0, "prefix_attn": 0, "layer_norm_eps": 1e-5}}
+    return {"bokorax": (bokorax, "bokorax"), "moondream2": (moondream, "moondream2")}
+
+
+def run_compare_bokorax(args, dtype, device) -> dict:
+    """Bokorax beside the Moondream decoder at equal sizes, through the same step function."""
+    return run_compare_design(args, dtype, device, "bokorax", BOKORAX_SIZES, bokorax_models)
 
 
 def run_compare_bogivik(args, dtype, device) -> dict:
@@ -674,14 +740,14 @@ def main() -> int:
                         help="with --workload: RuntimeConfig.tune_linears (time the vendor library's algorithms at warm-up)")
     parser.add_argument("--check", type=int, default=0,
                         help="with --workload: compare this many greedy requests with the plain implementation (for --layers 2)")
-    parser.add_argument("--workload", default="decode", choices=["decode", "waves256", "mixed48", "compare-vimesun", "compare-bogivik", "compare-letevik"],
+    parser.add_argument("--workload", default="decode", choices=["decode", "waves256", "mixed48", "compare-vimesun", "compare-bogivik", "compare-letevik", "compare-bokorax"],
                         help="decode: the benchmark's decode step (default); waves256 and mixed48 run requests through "
                              "InferenceEngine; compare-vimesun, compare-bogivik and compare-letevik measure that design beside the Moondream "
                              "decoder at equal sizes")
     parser.add_argument("--compare-sizes", default=None,
                         help="with --workload compare-*: which of its sizes, with commas between them "
                              "(default: all of them)")
-    parser.add_argument("--compare-model", default="both", choices=["both", "vimesun", "bogivik", "letevik", "moondream2"],
+    parser.add_argument("--compare-model", default="both", choices=["both", "vimesun", "bogivik", "letevik", "bokorax", "moondream2"],
                         help="with --workload compare-*: one of the two designs only (for profiling)")
     parser.add_argument("--compare-batches", default="1,8,64", help="with --workload compare-bogivik or compare-letevik: batch sizes of the decode steps")
     parser.add_argument("--skip-prefill", action="store_true", help="with --workload compare-bogivik or compare-letevik: decode steps only")
@@ -716,6 +782,9 @@ def main() -> int:
         return 0
     if args.workload == "compare-bogivik":
         print(json.dumps(run_compare_bogivik(args, dtype, device)))
+        return 0
+    if args.workload == "compare-bokorax":
+        print(json.dumps(run_compare_bokorax(args, dtype, device)))
         return 0
     if args.workload == "compare-letevik":
         print(json.dumps(run_compare_letevik(args, dtype, device)))

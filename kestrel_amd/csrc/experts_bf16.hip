@@ -8,8 +8,8 @@
 //  * gated (KA_ACT_GATED): weight rows 2j and 2j + 1 are gate and value of output j, as in every gated linear here.
 //
 // Both operands are rows that are contiguous along k, which is how v_mfma_f32_32x32x16_bf16 wants them: a lane loads 16
-// bytes of a weight row and of two activation rows per step straight from memory (a wave owns 32 weight rows and both
-// halves of the tile's 64 list rows, so a weight load serves two products; the activation rows are shared with the other
+// bytes of two weight rows and of two activation rows per step straight from memory (a wave owns 64 weight rows and both
+// halves of the tile's 64 list rows, so four loads feed four products; the activation rows are shared with the other
 // waves through the first-level cache). The weights are the row operand: a lane ends with outputs of ONE list row, four
 // neighbours at a time, so the pair of a gated output meets in a lane's registers.
 #include "ka_common.h"
@@ -20,7 +20,7 @@ typedef __attribute__((ext_vector_type(4))) __bf16 eb_bf16x4;
 typedef __attribute__((ext_vector_type(16))) float eb_floatx16;
 
 constexpr int EB_ROWS = 64;      // list rows a workgroup (and a tile of the list)
-constexpr int EB_COLS = 128;     // weight rows a workgroup: 32 a wave
+constexpr int EB_COLS = 256;     // weight rows a workgroup: 64 a wave
 
 __global__ void __launch_bounds__(256)
 experts_gemm_kernel(const bf16_t* __restrict__ a, long lda, int gather_div, const bf16_t* __restrict__ W, const int* __restrict__ sorted,
@@ -31,59 +31,67 @@ experts_gemm_kernel(const bf16_t* __restrict__ a, long lda, int gather_div, cons
     if (e < 0) return;                                   // (the unused end of the list)
     const int wave = threadIdx.x / KA_WAVE, lane = threadIdx.x % KA_WAVE;
     const int col = lane % 32, half = lane / 32;
-    const int o0 = blockIdx.x * EB_COLS + wave * 32;
+    const int o0 = blockIdx.x * EB_COLS + wave * 64;
     if (o0 >= N) return;                                 // (a whole wave; the kernel has no barrier)
     const int i0 = tile * EB_ROWS;
     const int p0 = sorted[i0 + col], p1 = sorted[i0 + 32 + col];
     // rows past the end, and unused rows of the list, are clamped for the loads and not stored
-    const bf16_t* wp = W + ((size_t)e * N + min(o0 + col, N - 1)) * K + half * 8;
+    const bf16_t* wp0 = W + ((size_t)e * N + min(o0 + col, N - 1)) * K + half * 8;
+    const bf16_t* wp1 = W + ((size_t)e * N + min(o0 + 32 + col, N - 1)) * K + half * 8;
     const long r0 = gather_div > 0 ? (long)max(p0, 0) / gather_div : (long)i0 + col;
     const long r1 = gather_div > 0 ? (long)max(p1, 0) / gather_div : (long)i0 + 32 + col;
     const bf16_t* ap0 = a + r0 * lda + half * 8;
     const bf16_t* ap1 = a + r1 * lda + half * 8;
-    eb_floatx16 acc0, acc1;
+    // acc[wb][rb]: weight rows o0 + 32 wb .., list rows i0 + 32 rb ..
+    eb_floatx16 acc[2][2];
 #pragma unroll
-    for (int i = 0; i < 16; ++i) acc0[i] = acc1[i] = 0.f;
-#pragma unroll 4
+    for (int i = 0; i < 16; ++i) acc[0][0][i] = acc[0][1][i] = acc[1][0][i] = acc[1][1][i] = 0.f;
+#pragma unroll 2
     for (int kk = 0; kk < K; kk += 16) {
-        const eb_bf16x8 w = *reinterpret_cast<const eb_bf16x8*>(wp + kk);
-        acc0 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(w, *reinterpret_cast<const eb_bf16x8*>(ap0 + kk), acc0, 0, 0, 0);
-        acc1 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(w, *reinterpret_cast<const eb_bf16x8*>(ap1 + kk), acc1, 0, 0, 0);
+        const eb_bf16x8 w0 = *reinterpret_cast<const eb_bf16x8*>(wp0 + kk);
+        const eb_bf16x8 w1 = *reinterpret_cast<const eb_bf16x8*>(wp1 + kk);
+        const eb_bf16x8 a0 = *reinterpret_cast<const eb_bf16x8*>(ap0 + kk);
+        const eb_bf16x8 a1 = *reinterpret_cast<const eb_bf16x8*>(ap1 + kk);
+        acc[0][0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(w0, a0, acc[0][0], 0, 0, 0);
+        acc[0][1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(w0, a1, acc[0][1], 0, 0, 0);
+        acc[1][0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(w1, a0, acc[1][0], 0, 0, 0);
+        acc[1][1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(w1, a1, acc[1][1], 0, 0, 0);
     }
     const bool gated = ka_act_gated(act);
 #pragma unroll
-    for (int blk = 0; blk < 2; ++blk) {
+    for (int both = 0; both < 4; ++both) {
+        const int blk = both & 1, wb = both >> 1;
         const int p = blk ? p1 : p0;
         if (p < 0) continue;
-        const eb_floatx16& acc = blk ? acc1 : acc0;
+        const eb_floatx16& acc_here = acc[wb][blk];
         const long row = scatter ? (long)p : (long)i0 + blk * 32 + col;
-        // register i: weight row o0 + (i / 4) * 8 + half * 4 + i % 4 of the lane's list row
+        // register i: weight row o0 + 32 wb + (i / 4) * 8 + half * 4 + i % 4 of the lane's list row
 #pragma unroll
         for (int g4 = 0; g4 < 4; ++g4) {
-            const int o = o0 + g4 * 8 + half * 4;
+            const int o = o0 + wb * 32 + g4 * 8 + half * 4;
             if (gated) {
                 if (o + 3 < N) {
                     eb_bf16x2 y;
-                    y[0] = (bf16_t)(ka_activate_fast(act, acc[g4 * 4]) * acc[g4 * 4 + 1]);
-                    y[1] = (bf16_t)(ka_activate_fast(act, acc[g4 * 4 + 2]) * acc[g4 * 4 + 3]);
+                    y[0] = (bf16_t)(ka_activate_fast(act, acc_here[g4 * 4]) * acc_here[g4 * 4 + 1]);
+                    y[1] = (bf16_t)(ka_activate_fast(act, acc_here[g4 * 4 + 2]) * acc_here[g4 * 4 + 3]);
                     *reinterpret_cast<eb_bf16x2*>(reinterpret_cast<bf16_t*>(out) + row * ldo + o / 2) = y;
                 } else if (o + 1 < N) {
-                    reinterpret_cast<bf16_t*>(out)[row * ldo + o / 2] = (bf16_t)(ka_activate_fast(act, acc[g4 * 4]) * acc[g4 * 4 + 1]);
+                    reinterpret_cast<bf16_t*>(out)[row * ldo + o / 2] = (bf16_t)(ka_activate_fast(act, acc_here[g4 * 4]) * acc_here[g4 * 4 + 1]);
                 }
             } else if (out_f32) {
                 float* op = reinterpret_cast<float*>(out) + row * ldo + o;
                 if (o + 3 < N) {
-                    *reinterpret_cast<float4*>(op) = make_float4(acc[g4 * 4], acc[g4 * 4 + 1], acc[g4 * 4 + 2], acc[g4 * 4 + 3]);
+                    *reinterpret_cast<float4*>(op) = make_float4(acc_here[g4 * 4], acc_here[g4 * 4 + 1], acc_here[g4 * 4 + 2], acc_here[g4 * 4 + 3]);
                 } else {
 #pragma unroll
                     for (int x = 0; x < 4; ++x)
-                        if (o + x < N) op[x] = acc[g4 * 4 + x];
+                        if (o + x < N) op[x] = acc_here[g4 * 4 + x];
                 }
             } else {
                 bf16_t* op = reinterpret_cast<bf16_t*>(out) + row * ldo + o;
 #pragma unroll
                 for (int x = 0; x < 4; ++x)
-                    if (o + x < N) op[x] = (bf16_t)(ka_act_base(act) ? ka_activate_fast(act, acc[g4 * 4 + x]) : acc[g4 * 4 + x]);
+                    if (o + x < N) op[x] = (bf16_t)(ka_act_base(act) ? ka_activate_fast(act, acc_here[g4 * 4 + x]) : acc_here[g4 * 4 + x]);
             }
         }
     }

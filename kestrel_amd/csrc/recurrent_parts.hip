@@ -83,7 +83,8 @@ struct DecayArgs {
     float eps;
 };
 
-template <typename T, int NI>
+// FULL: d is a multiple of NI (no thread's range of key channels ends early) and of 4 (the LDS rows are read four at a time).
+template <typename T, int NI, bool FULL>
 __global__ void __launch_bounds__(1024) decayed_memory_kernel(DecayArgs a) {
     extern __shared__ float sm[];
     const int head = blockIdx.x, row = blockIdx.y, tid = threadIdx.x;
@@ -102,8 +103,8 @@ __global__ void __launch_bounds__(1024) decayed_memory_kernel(DecayArgs a) {
     float* ks = rs + (size_t)TB * d;
     float* ws = ks + (size_t)TB * d;
     float* vs = ws + (size_t)TB * d;
-    float* po = vs + (size_t)TB * d;        // [TB][P][d]
-    float* cs = po + (size_t)TB * P * d;    // [TB]: sum_i r_i u_i k_i
+    float* bs = vs + (size_t)TB * d;        // [TB][d]: r_i u_i k_i, whose sum over i is the bonus term's factor
+    float* po = bs + (size_t)TB * d;        // [TB][P][d]
     const int j = tid % d, p = tid / d;
     const bool works = p < P;
     const int i0 = p * NI;
@@ -126,13 +127,9 @@ __global__ void __launch_bounds__(1024) decayed_memory_kernel(DecayArgs a) {
             ks[e] = ka_to_float(kp[at]);
             vs[e] = ka_to_float(vp[at]);
             ws[e] = expf(-expf(a.pre[(size_t)(tb + tt) * a.H * d + (size_t)head * d + c]));
+            bs[e] = rs[e] * up[c] * ks[e];
         }
         __syncthreads();
-        if (tid < nb) {
-            float c = 0.f;
-            for (int i = 0; i < d; ++i) c = fmaf(rs[tid * d + i] * up[i], ks[tid * d + i], c);
-            cs[tid] = c;
-        }
         if (works) {
             for (int tt = 0; tt < nb; ++tt) {
                 const float vj = vs[tt * d + j];
@@ -140,11 +137,28 @@ __global__ void __launch_bounds__(1024) decayed_memory_kernel(DecayArgs a) {
                 const float* k_t = ks + tt * d + i0;
                 const float* w_t = ws + tt * d + i0;
                 float acc = 0.f;
+                if constexpr (FULL) {
 #pragma unroll
-                for (int ii = 0; ii < NI; ++ii) {
-                    if (i0 + ii < d) {
-                        acc = fmaf(r_t[ii], S[ii], acc);
-                        S[ii] = fmaf(w_t[ii], S[ii], k_t[ii] * vj);
+                    for (int ii = 0; ii < NI; ii += 4) {
+                        const float4 r4 = *reinterpret_cast<const float4*>(r_t + ii);
+                        const float4 k4 = *reinterpret_cast<const float4*>(k_t + ii);
+                        const float4 w4 = *reinterpret_cast<const float4*>(w_t + ii);
+                        acc = fmaf(r4.x, S[ii], acc);
+                        S[ii] = fmaf(w4.x, S[ii], k4.x * vj);
+                        acc = fmaf(r4.y, S[ii + 1], acc);
+                        S[ii + 1] = fmaf(w4.y, S[ii + 1], k4.y * vj);
+                        acc = fmaf(r4.z, S[ii + 2], acc);
+                        S[ii + 2] = fmaf(w4.z, S[ii + 2], k4.z * vj);
+                        acc = fmaf(r4.w, S[ii + 3], acc);
+                        S[ii + 3] = fmaf(w4.w, S[ii + 3], k4.w * vj);
+                    }
+                } else {
+#pragma unroll
+                    for (int ii = 0; ii < NI; ++ii) {
+                        if (i0 + ii < d) {
+                            acc = fmaf(r_t[ii], S[ii], acc);
+                            S[ii] = fmaf(w_t[ii], S[ii], k_t[ii] * vj);
+                        }
                     }
                 }
                 po[((size_t)tt * P + p) * d + j] = acc;
@@ -154,13 +168,17 @@ __global__ void __launch_bounds__(1024) decayed_memory_kernel(DecayArgs a) {
         // read-outs of the block: a wave per token, lanes over the value channels
         for (int tt = wave; tt < nb; tt += n_waves) {
             float o[4];
-            float ss = 0.f;
+            float ss = 0.f, bonus = 0.f;
+#pragma unroll
+            for (int q = 0; q < 4; ++q)
+                if (lane + q * KA_WAVE < d) bonus += bs[tt * d + lane + q * KA_WAVE];
+            bonus = ka_wave_sum(bonus);
 #pragma unroll
             for (int q = 0; q < 4; ++q) {
                 const int c = lane + q * KA_WAVE;
                 o[q] = 0.f;
                 if (c < d) {
-                    float y = cs[tt] * vs[tt * d + c];
+                    float y = bonus * vs[tt * d + c];
                     for (int pp = 0; pp < P; ++pp) y += po[((size_t)tt * P + pp) * d + c];
                     o[q] = y;
                     ss = fmaf(y, y, ss);
@@ -194,7 +212,7 @@ __global__ void __launch_bounds__(1024) decayed_memory_kernel(DecayArgs a) {
 // How the kernel cuts a head of d channels: NI state entries a thread, `parts` threads a value channel.
 static bool decay_shape(int d, int* ni, int* parts) {
     if (d <= 0 || d > 256) return false;
-    for (int cand : {16, 32, 64}) {
+    for (int cand : {4, 8, 16, 32, 64}) {
         const int pp = (d + cand - 1) / cand;
         if ((long)pp * d <= 1024) {
             *ni = cand;
@@ -222,18 +240,21 @@ KA_API int ka_decayed_memory(const void* r, const void* k, const void* v, const 
     KA_CHECK(state_stride >= (long)H * d * d + (x ? dim : 0), "%s: the state rows are too short", who);
     KA_CHECK(H <= 65535 && n_rows <= 65535, "%s: too many heads or rows", who);
     if (n_rows == 0) return 0;
-    int block_tokens = 32768 / (d * 4 * (4 + parts));
+    int block_tokens = 49152 / (d * 4 * (5 + parts));
     block_tokens = block_tokens < 1 ? 1 : (block_tokens > 16 ? 16 : block_tokens);
     const int threads = ((parts * d + KA_WAVE - 1) / KA_WAVE) * KA_WAVE;
-    const size_t lds = ((size_t)block_tokens * d * (4 + parts) + block_tokens) * sizeof(float);
+    const size_t lds = (size_t)block_tokens * d * (5 + parts) * sizeof(float);
+    const bool full = d % ni == 0 && d % 4 == 0;
     DecayArgs a{r, k, v, gate, stride, pre, u, gain, state, state_stride, x, dim, cu_q, row_slot, out, out_stride, H, d, block_tokens, parts, eps};
     dim3 grid(H, n_rows);
-#define RP_LAUNCH(T, NI) hipLaunchKernelGGL((decayed_memory_kernel<T, NI>), grid, dim3(threads), lds, stream, a)
-    if (dtype == KA_F32) {
-        if (ni == 16) RP_LAUNCH(float, 16); else if (ni == 32) RP_LAUNCH(float, 32); else RP_LAUNCH(float, 64);
-    } else {
-        if (ni == 16) RP_LAUNCH(bf16_t, 16); else if (ni == 32) RP_LAUNCH(bf16_t, 32); else RP_LAUNCH(bf16_t, 64);
+#define RP_LAUNCH(T, NI)                                                                                             \
+    if (ni == NI) {                                                                                                  \
+        if (full) hipLaunchKernelGGL((decayed_memory_kernel<T, NI, true>), grid, dim3(threads), lds, stream, a);     \
+        else hipLaunchKernelGGL((decayed_memory_kernel<T, NI, false>), grid, dim3(threads), lds, stream, a);         \
     }
+#define RP_LAUNCH_ALL(T) RP_LAUNCH(T, 4) RP_LAUNCH(T, 8) RP_LAUNCH(T, 16) RP_LAUNCH(T, 32) RP_LAUNCH(T, 64)
+    if (dtype == KA_F32) { RP_LAUNCH_ALL(float) } else { RP_LAUNCH_ALL(bf16_t) }
+#undef RP_LAUNCH_ALL
 #undef RP_LAUNCH
     KA_LAUNCH_CHECK();
     return 0;

@@ -16,7 +16,7 @@ class RoutedExperts(FeedForward):
     """``sum over the chosen k of weight_k * expert_k(h) [+ sigmoid(shared.sg h) * shared(h)]``.
 
     Every expert is ``down(act(gate h) * (up h))`` without biases (tensors ``e<i>.gate.weight`` and so on). The router
-    (``router.weight`` ``[n_experts + n_identity, dim]``) runs in fp32; how its scores become a choice and weights is
+    (``router.weight`` ``[n_experts + n_identity, dim]``) writes fp32 logits from fp32 sums, and the choice is made in fp32; how its scores become a choice and weights is
     ``RoutedExpertsSpec``'s text. The router's last ``n_identity`` outputs are identity experts: their output is ``h``.
     The shared expert (``shared.*``) has the experts' form and a hidden size of its own; its gate ``shared.sg.weight``
     ``[1, dim]`` rides as one more row of the router's linear.
@@ -73,10 +73,13 @@ class RoutedExperts(FeedForward):
         self.pairs = torch.stack([pair_rows(tensors[f"e{e}.gate.weight"].to(device), tensors[f"e{e}.up.weight"].to(device))
                                   for e in range(spec.n_experts)]).contiguous()
         self.down = torch.stack([tensors[f"e{e}.down.weight"].to(device) for e in range(spec.n_experts)]).contiguous()
-        rows = [tensors["router.weight"].to(device=device, dtype=torch.float32)]
+        # The router's rows stay in the type they are held in: products of bf16 numbers are exact in fp32 and every linear
+        # kernel sums in fp32, so a bf16 run computes the router's sums in 32 bits from the rounded input, as an fp32 run does
+        # from its own. The shared expert's gate rides as one more row.
+        rows = [tensors["router.weight"].to(device)]
         if self.gated_shared:
-            rows.append(tensors["shared.sg.weight"].to(device=device, dtype=torch.float32).reshape(1, spec.dim))
-        self.router = torch.cat(rows, dim=0).contiguous()          # fp32: the router's sums are fp32 whatever the run
+            rows.append(tensors["shared.sg.weight"].to(device=device, dtype=rows[0].dtype).reshape(1, spec.dim))
+        self.router = torch.cat(rows, dim=0).contiguous()
         self.correction = tensors["correction"].to(device=device, dtype=torch.float32).contiguous()
         if self.shared:
             self.shared_pairs = pair_rows(tensors["shared.gate.weight"].to(device), tensors["shared.up.weight"].to(device))
@@ -89,7 +92,7 @@ class RoutedExperts(FeedForward):
         ws = batch.workspace
         top, E = spec.top, spec.n_experts
         logits = ws.get("experts.logits", (n, self.router.shape[0]), torch.float32)
-        core.linear_generic(h, self.router, None, logits)
+        linear(h, self.router, None, logits)
         chosen = ws.get("experts.chosen", (n, top), torch.int32)
         weights = ws.get("experts.weights", (n, top), torch.float32)
         core.route(logits, self.n_outputs, self.correction, top, spec.n_groups, spec.keep_groups, spec.scale, chosen, weights)
