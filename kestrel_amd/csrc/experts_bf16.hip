@@ -1,16 +1,16 @@
 // The linears of routed experts on the matrix cores (bf16): the pairs (token, choice) of a step come listed by expert, in
-// runs that start on multiples of 64 rows of the list (ka_experts_sort), and a workgroup multiplies one tile of 64 list
-// rows by 128 rows of its expert's weights: out[row] = act(a[row'] W_e^T).
+// runs that start on multiples of 128 rows of the list (ka_experts_sort), and a workgroup multiplies one tile of 128 list
+// rows by 256 rows of its expert's weights: out[row] = act(a[row'] W_e^T).
 //
 //  * the first linear gathers: list row i holds pair p = sorted[i] (-1: an unused row), whose input is row p / gather_div
 //    of `a`; its output goes to row i of `out` (the hidden rows stay in list order);
 //  * the second linear scatters: its input is row i of `a`, its output goes to row p of `out`;
 //  * gated (KA_ACT_GATED): weight rows 2j and 2j + 1 are gate and value of output j, as in every gated linear here.
 //
-// Both operands are rows that are contiguous along k, which is how v_mfma_f32_32x32x16_bf16 wants them: a lane loads 16
-// bytes of two weight rows and of two activation rows per step straight from memory (a wave owns 64 weight rows and both
-// halves of the tile's 64 list rows, so four loads feed four products; the activation rows are shared with the other
-// waves through the first-level cache). The weights are the row operand: a lane ends with outputs of ONE list row, four
+// Both operands are rows that are contiguous along k, which is how v_mfma_f32_32x32x16_bf16 wants them: a lane loads 64
+// bytes in a row of two weight rows and of four activation rows per slab of 64 channels, straight from memory (a wave
+// owns 64 weight rows and all of the tile's 128 list rows: 24 loads feed 32 products; the activation rows are shared
+// with the other waves through the first-level cache, and a weight row's line is used up by the lane pair that asked). The weights are the row operand: a lane ends with outputs of ONE list row, four
 // neighbours at a time, so the pair of a gated output meets in a lane's registers.
 #include "ka_common.h"
 
@@ -19,8 +19,9 @@ typedef __attribute__((ext_vector_type(2))) __bf16 eb_bf16x2;
 typedef __attribute__((ext_vector_type(4))) __bf16 eb_bf16x4;
 typedef __attribute__((ext_vector_type(16))) float eb_floatx16;
 
-constexpr int EB_ROWS = 64;      // list rows a workgroup (and a tile of the list)
-constexpr int EB_COLS = 256;     // weight rows a workgroup: 64 a wave
+constexpr int EB_ROWS = 128;     // list rows a workgroup (and a tile of the list): four blocks of 32
+constexpr int EB_COLS = 256;     // weight rows a workgroup: 64 a wave, two blocks of 32
+constexpr int EB_SLAB = 64;      // channels of k a lane's loads cover at a time: with its partner lane a whole 128-byte line
 
 __global__ void __launch_bounds__(256)
 experts_gemm_kernel(const bf16_t* __restrict__ a, long lda, int gather_div, const bf16_t* __restrict__ W, const int* __restrict__ sorted,
@@ -34,64 +35,112 @@ experts_gemm_kernel(const bf16_t* __restrict__ a, long lda, int gather_div, cons
     const int o0 = blockIdx.x * EB_COLS + wave * 64;
     if (o0 >= N) return;                                 // (a whole wave; the kernel has no barrier)
     const int i0 = tile * EB_ROWS;
-    const int p0 = sorted[i0 + col], p1 = sorted[i0 + 32 + col];
-    // rows past the end, and unused rows of the list, are clamped for the loads and not stored
-    const bf16_t* wp0 = W + ((size_t)e * N + min(o0 + col, N - 1)) * K + half * 8;
-    const bf16_t* wp1 = W + ((size_t)e * N + min(o0 + 32 + col, N - 1)) * K + half * 8;
-    const long r0 = gather_div > 0 ? (long)max(p0, 0) / gather_div : (long)i0 + col;
-    const long r1 = gather_div > 0 ? (long)max(p1, 0) / gather_div : (long)i0 + 32 + col;
-    const bf16_t* ap0 = a + r0 * lda + half * 8;
-    const bf16_t* ap1 = a + r1 * lda + half * 8;
-    // acc[wb][rb]: weight rows o0 + 32 wb .., list rows i0 + 32 rb ..
-    eb_floatx16 acc[2][2];
+    int pr[4];
 #pragma unroll
-    for (int i = 0; i < 16; ++i) acc[0][0][i] = acc[0][1][i] = acc[1][0][i] = acc[1][1][i] = 0.f;
-#pragma unroll 2
-    for (int kk = 0; kk < K; kk += 16) {
-        const eb_bf16x8 w0 = *reinterpret_cast<const eb_bf16x8*>(wp0 + kk);
-        const eb_bf16x8 w1 = *reinterpret_cast<const eb_bf16x8*>(wp1 + kk);
-        const eb_bf16x8 a0 = *reinterpret_cast<const eb_bf16x8*>(ap0 + kk);
-        const eb_bf16x8 a1 = *reinterpret_cast<const eb_bf16x8*>(ap1 + kk);
-        acc[0][0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(w0, a0, acc[0][0], 0, 0, 0);
-        acc[0][1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(w0, a1, acc[0][1], 0, 0, 0);
-        acc[1][0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(w1, a0, acc[1][0], 0, 0, 0);
-        acc[1][1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(w1, a1, acc[1][1], 0, 0, 0);
+    for (int rb = 0; rb < 4; ++rb) pr[rb] = sorted[i0 + rb * 32 + col];
+    // rows past the end, and unused rows of the list, are clamped for the loads and not stored
+    const bf16_t* wp[2];
+#pragma unroll
+    for (int wb = 0; wb < 2; ++wb) wp[wb] = W + ((size_t)e * N + min(o0 + wb * 32 + col, N - 1)) * K;
+    const bf16_t* ap[4];
+#pragma unroll
+    for (int rb = 0; rb < 4; ++rb)
+        ap[rb] = a + (gather_div > 0 ? (long)max(pr[rb], 0) / gather_div : (long)i0 + rb * 32 + col) * lda;
+    // acc[wb][rb]: weight rows o0 + 32 wb .., list rows i0 + 32 rb ..
+    eb_floatx16 acc[2][4];
+#pragma unroll
+    for (int wb = 0; wb < 2; ++wb)
+#pragma unroll
+        for (int rb = 0; rb < 4; ++rb)
+#pragma unroll
+            for (int i = 0; i < 16; ++i) acc[wb][rb][i] = 0.f;
+    // Slabs of 64 channels: a lane reads the 32 channels [32 half, 32 half + 32) of its rows, 64 bytes in a row, and feeds
+    // them to four products, eight channels each. Which channels meet in a product does not matter as long as both
+    // operands agree, and they do: piece m of half h is the channels 32 h + 8 m .. + 7 of the slab for both.
+    // (the next slab's loads are asked for before the products of this one: a wave has its SIMD to itself, and nothing
+    // else would hide their way from memory)
+    int kk = 0;
+    eb_bf16x8 w[2][4], x[4][4];
+    auto load = [&](int at, eb_bf16x8 (&wn)[2][4], eb_bf16x8 (&xn)[4][4]) {
+#pragma unroll
+        for (int wb = 0; wb < 2; ++wb)
+#pragma unroll
+            for (int m = 0; m < 4; ++m) wn[wb][m] = *reinterpret_cast<const eb_bf16x8*>(wp[wb] + at + half * 32 + m * 8);
+#pragma unroll
+        for (int rb = 0; rb < 4; ++rb)
+#pragma unroll
+            for (int m = 0; m < 4; ++m) xn[rb][m] = *reinterpret_cast<const eb_bf16x8*>(ap[rb] + at + half * 32 + m * 8);
+    };
+    if (EB_SLAB <= K) load(0, w, x);
+    for (; kk + EB_SLAB <= K; kk += EB_SLAB) {
+        eb_bf16x8 wn[2][4], xn[4][4];
+        const bool more = kk + 2 * EB_SLAB <= K;
+        if (more) load(kk + EB_SLAB, wn, xn);
+#pragma unroll
+        for (int m = 0; m < 4; ++m)
+#pragma unroll
+            for (int wb = 0; wb < 2; ++wb)
+#pragma unroll
+                for (int rb = 0; rb < 4; ++rb)
+                    acc[wb][rb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(w[wb][m], x[rb][m], acc[wb][rb], 0, 0, 0);
+        if (more) {
+#pragma unroll
+            for (int m = 0; m < 4; ++m) {
+#pragma unroll
+                for (int wb = 0; wb < 2; ++wb) w[wb][m] = wn[wb][m];
+#pragma unroll
+                for (int rb = 0; rb < 4; ++rb) x[rb][m] = xn[rb][m];
+            }
+        }
+    }
+    for (; kk < K; kk += 16) {                            // (what is left of a K that is no multiple of 64: steps of 16)
+        eb_bf16x8 wt[2], xt[4];
+#pragma unroll
+        for (int wb = 0; wb < 2; ++wb) wt[wb] = *reinterpret_cast<const eb_bf16x8*>(wp[wb] + kk + half * 8);
+#pragma unroll
+        for (int rb = 0; rb < 4; ++rb) xt[rb] = *reinterpret_cast<const eb_bf16x8*>(ap[rb] + kk + half * 8);
+#pragma unroll
+        for (int wb = 0; wb < 2; ++wb)
+#pragma unroll
+            for (int rb = 0; rb < 4; ++rb) acc[wb][rb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(wt[wb], xt[rb], acc[wb][rb], 0, 0, 0);
     }
     const bool gated = ka_act_gated(act);
 #pragma unroll
-    for (int both = 0; both < 4; ++both) {
-        const int blk = both & 1, wb = both >> 1;
-        const int p = blk ? p1 : p0;
+    for (int rb = 0; rb < 4; ++rb) {
+        const int p = pr[rb];
         if (p < 0) continue;
-        const eb_floatx16& acc_here = acc[wb][blk];
-        const long row = scatter ? (long)p : (long)i0 + blk * 32 + col;
-        // register i: weight row o0 + 32 wb + (i / 4) * 8 + half * 4 + i % 4 of the lane's list row
+        const long row = scatter ? (long)p : (long)i0 + rb * 32 + col;
 #pragma unroll
-        for (int g4 = 0; g4 < 4; ++g4) {
-            const int o = o0 + wb * 32 + g4 * 8 + half * 4;
-            if (gated) {
-                if (o + 3 < N) {
-                    eb_bf16x2 y;
-                    y[0] = (bf16_t)(ka_activate_fast(act, acc_here[g4 * 4]) * acc_here[g4 * 4 + 1]);
-                    y[1] = (bf16_t)(ka_activate_fast(act, acc_here[g4 * 4 + 2]) * acc_here[g4 * 4 + 3]);
-                    *reinterpret_cast<eb_bf16x2*>(reinterpret_cast<bf16_t*>(out) + row * ldo + o / 2) = y;
-                } else if (o + 1 < N) {
-                    reinterpret_cast<bf16_t*>(out)[row * ldo + o / 2] = (bf16_t)(ka_activate_fast(act, acc_here[g4 * 4]) * acc_here[g4 * 4 + 1]);
-                }
-            } else if (out_f32) {
-                float* op = reinterpret_cast<float*>(out) + row * ldo + o;
-                if (o + 3 < N) {
-                    *reinterpret_cast<float4*>(op) = make_float4(acc_here[g4 * 4], acc_here[g4 * 4 + 1], acc_here[g4 * 4 + 2], acc_here[g4 * 4 + 3]);
+        for (int wb = 0; wb < 2; ++wb) {
+            const eb_floatx16& acc_here = acc[wb][rb];
+            // register i: weight row o0 + 32 wb + (i / 4) * 8 + half * 4 + i % 4 of the lane's list row
+#pragma unroll
+            for (int g4 = 0; g4 < 4; ++g4) {
+                const int o = o0 + wb * 32 + g4 * 8 + half * 4;
+                if (gated) {
+                    if (o + 3 < N) {
+                        eb_bf16x2 y;
+                        y[0] = (bf16_t)(ka_activate_fast(act, acc_here[g4 * 4]) * acc_here[g4 * 4 + 1]);
+                        y[1] = (bf16_t)(ka_activate_fast(act, acc_here[g4 * 4 + 2]) * acc_here[g4 * 4 + 3]);
+                        *reinterpret_cast<eb_bf16x2*>(reinterpret_cast<bf16_t*>(out) + row * ldo + o / 2) = y;
+                    } else if (o + 1 < N) {
+                        reinterpret_cast<bf16_t*>(out)[row * ldo + o / 2] = (bf16_t)(ka_activate_fast(act, acc_here[g4 * 4]) * acc_here[g4 * 4 + 1]);
+                    }
+                } else if (out_f32) {
+                    float* op = reinterpret_cast<float*>(out) + row * ldo + o;
+                    if (o + 3 < N) {
+                        *reinterpret_cast<float4*>(op) = make_float4(acc_here[g4 * 4], acc_here[g4 * 4 + 1], acc_here[g4 * 4 + 2], acc_here[g4 * 4 + 3]);
+                    } else {
+#pragma unroll
+                        for (int x = 0; x < 4; ++x)
+                            if (o + x < N) op[x] = acc_here[g4 * 4 + x];
+                    }
                 } else {
+                    bf16_t* op = reinterpret_cast<bf16_t*>(out) + row * ldo + o;
 #pragma unroll
                     for (int x = 0; x < 4; ++x)
-                        if (o + x < N) op[x] = acc_here[g4 * 4 + x];
+                        if (o + x < N) op[x] = (bf16_t)(ka_act_base(act) ? ka_activate_fast(act, acc_here[g4 * 4 + x]) : acc_here[g4 * 4 + x]);
                 }
-            } else {
-                bf16_t* op = reinterpret_cast<bf16_t*>(out) + row * ldo + o;
-#pragma unroll
-                for (int x = 0; x < 4; ++x)
-                    if (o + x < N) op[x] = (bf16_t)(ka_act_base(act) ? ka_activate_fast(act, acc_here[g4 * 4 + x]) : acc_here[g4 * 4 + x]);
             }
         }
     }

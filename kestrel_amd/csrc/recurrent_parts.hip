@@ -54,58 +54,63 @@ KA_API int ka_token_shift(const float* x, const float* kept, long kept_stride, c
 //     S_ij <- w_i S_ij + k_i v_j
 // then o is divided by its root mean square over the head (eps), multiplied by gain and by the gate.
 //
-// A workgroup owns one head of one row and walks over the row's tokens of this step, whatever they are (a prompt, a
-// portion, one token). Thread (p, j) keeps the NI entries S[p NI .. p NI + NI - 1][j] in registers. Tokens are taken
-// in blocks: r, k, w and v of a block are staged in LDS in fp32 (w computed there), the threads then run the
-// recurrence over the block's tokens with no exchange between them but the LDS reads, leave their partial read-outs
-// in LDS, and the read-outs of the block are summed, normalised, gated and stored a wave per token. Every token's
-// arithmetic is the same wherever a step was cut. A row without a request (slot < 0) writes zeros.
-// The workgroup of head 0 also keeps the stream's last row of the portion for the next step's token shift.
+// Two launches. The first walks over every row's tokens of this step, whatever they are (a prompt, a portion, one
+// token), and leaves the read-outs o in fp32. The columns j of S are independent of each other, so a head is dealt out
+// over workgroups by slices of value channels (blockIdx.z) as well as over threads: thread (p, j) of a workgroup keeps
+// the NI entries S[p NI .. p NI + NI - 1][j] in registers. Tokens are taken in blocks: r, k, w, v and u r k of a block are
+// staged in LDS in fp32 (w computed there; the next block's numbers are already on their way from memory), the threads
+// then run the recurrence over the block's tokens with no exchange between them but the LDS reads, leave their partial
+// read-outs in LDS, and the partial read-outs of the block are summed a wave per token. Every token's arithmetic is the
+// same wherever a step was cut. What a token costs is instructions (a hundred and fifty a wave with a quarter of a head of
+// 64 a thread, counted on the GPU), so the fast form (heads that are multiples of 16 channels) gives a thread four key
+// channels of one value channel, sixteen value channels a workgroup.
+// The second launch normalises, a wave per (token, head). A row without a request (slot < 0) gets zeros.
+// The workgroup of head 0, slice 0 also keeps the stream's last row of the portion for the next step's token shift.
 // ----------------------------------------------------------------------------
 struct DecayArgs {
     const void* r;
     const void* k;
     const void* v;
-    const void* gate;
-    long stride;            // of the rows of r, k, v and gate
+    long stride;            // of the rows of r, k and v
     const float* pre;       // [n, H d]
     const float* u;         // [H d]
-    const float* gain;      // [H d]
     float* state;           // [slots, state_stride]: S [H, d, d], then the kept row [dim]
     long state_stride;
     const float* x;         // the stream [n, dim] (the kept row comes from it), or null
     int dim;
     const int* cu_q;
     const int* row_slot;
-    void* out;
-    long out_stride;
-    int H, d, block_tokens, parts;
-    float eps;
+    float* raw;             // [n, H d]: the read-outs before their norm
+    int H, d, block_tokens, parts, slice;       // slice: value channels a workgroup
 };
 
-// FULL: d is a multiple of NI (no thread's range of key channels ends early) and of 4 (the LDS rows are read four at a time).
-template <typename T, int NI, bool FULL>
-__global__ void __launch_bounds__(1024) decayed_memory_kernel(DecayArgs a) {
+constexpr int RP_SLICE = 16;        // value channels a workgroup of the fast form (half as many for heads above 128 channels)
+
+// FAST: d is a multiple of 16; NI = 4 key channels a thread (read from LDS four at a time), RP_SLICE value channels a
+// workgroup. Otherwise any d, the whole head a workgroup.
+template <typename T, int NI, bool FAST>
+__global__ void __launch_bounds__(!FAST && NI == 64 ? 1024 : 512) decayed_memory_kernel(DecayArgs a) {
     extern __shared__ float sm[];
     const int head = blockIdx.x, row = blockIdx.y, tid = threadIdx.x;
-    const int d = a.d, TB = a.block_tokens, P = a.parts;
+    const int d = a.d, TB = a.block_tokens, P = a.parts, dj = a.slice;
+    const int j0 = blockIdx.z * dj;
     const int t0 = a.cu_q[row], t1 = a.cu_q[row + 1];
     if (t0 >= t1) return;
     const int slot = a.row_slot[row];
     const int wave = tid / KA_WAVE, lane = tid % KA_WAVE, n_waves = blockDim.x / KA_WAVE;
-    T* out = reinterpret_cast<T*>(a.out);
     if (slot < 0) {
-        for (int e = tid; e < (t1 - t0) * d; e += blockDim.x)
-            out[(size_t)(t0 + e / d) * a.out_stride + (size_t)head * d + e % d] = ka_from_float<T>(0.f);
+        for (int e = tid; e < (t1 - t0) * dj; e += blockDim.x)
+            a.raw[(size_t)(t0 + e / dj) * a.H * d + (size_t)head * d + j0 + e % dj] = 0.f;
         return;
     }
     float* rs = sm;                         // [TB][d]
     float* ks = rs + (size_t)TB * d;
     float* ws = ks + (size_t)TB * d;
-    float* vs = ws + (size_t)TB * d;
-    float* bs = vs + (size_t)TB * d;        // [TB][d]: r_i u_i k_i, whose sum over i is the bonus term's factor
-    float* po = bs + (size_t)TB * d;        // [TB][P][d]
-    const int j = tid % d, p = tid / d;
+    float* bs = ws + (size_t)TB * d;        // [TB][d]: r_i u_i k_i, whose sum over i is the bonus term's factor
+    float* vs = bs + (size_t)TB * d;        // [TB][dj]
+    float* po = vs + (size_t)TB * dj;       // [TB][P][dj]
+    const int jl = tid % dj, p = tid / dj;
+    const int j = j0 + jl;
     const bool works = p < P;
     const int i0 = p * NI;
     float* S_mem = a.state + (size_t)slot * a.state_stride + (size_t)head * d * d;
@@ -115,106 +120,160 @@ __global__ void __launch_bounds__(1024) decayed_memory_kernel(DecayArgs a) {
     const T* rp = reinterpret_cast<const T*>(a.r) + (size_t)head * d;
     const T* kp = reinterpret_cast<const T*>(a.k) + (size_t)head * d;
     const T* vp = reinterpret_cast<const T*>(a.v) + (size_t)head * d;
-    const T* gp = reinterpret_cast<const T*>(a.gate) + (size_t)head * d;
     const float* up = a.u + (size_t)head * d;
-    const float* gain = a.gain + (size_t)head * d;
+    // what a thread fetches of a block: its elements e = tid + m * threads of r, k, the decay's pre-activation and (of the
+    // slice's channels) v. The next block's are asked for before the current block is computed.
+    constexpr int RP_FETCH = FAST ? 4 : (NI == 64 ? 2 : 8);      // (the host sizes the block so that a thread has at most this many)
+    T fr[RP_FETCH], fk[RP_FETCH], fv[RP_FETCH];
+    float fw[RP_FETCH];
+    auto fetch = [&](int tb) {
+        const int nb = min(TB, t1 - tb);
+#pragma unroll
+        for (int m = 0; m < RP_FETCH; ++m) {
+            const int e = tid + m * (int)blockDim.x;
+            if (e < nb * d) {
+                const int tt = e / d, c = e % d;
+                const size_t at = (size_t)(tb + tt) * a.stride + c;
+                fr[m] = rp[at];
+                fk[m] = kp[at];
+                fw[m] = a.pre[(size_t)(tb + tt) * a.H * d + (size_t)head * d + c];
+            }
+            if (e < nb * dj) fv[m] = vp[(size_t)(tb + e / dj) * a.stride + j0 + e % dj];
+        }
+    };
+    // This wave's LDS writes done, then everybody's: what __syncthreads() does too, but that one also waits for every load
+    // and store in flight, which is the next block's numbers on their way from memory and the read-outs on their way there.
+    auto lds_barrier = [&]() {
+        __builtin_amdgcn_s_waitcnt(0xc07f);      // lgkmcnt(0), the other counters at their maximum
+        asm volatile("" ::: "memory");
+        __builtin_amdgcn_s_barrier();
+        asm volatile("" ::: "memory");
+    };
+    fetch(t0);
     for (int tb = t0; tb < t1; tb += TB) {
         const int nb = min(TB, t1 - tb);
-        for (int e = tid; e < nb * d; e += blockDim.x) {
-            const int tt = e / d, c = e % d;
-            const size_t at = (size_t)(tb + tt) * a.stride + c;
-            rs[e] = ka_to_float(rp[at]);
-            ks[e] = ka_to_float(kp[at]);
-            vs[e] = ka_to_float(vp[at]);
-            ws[e] = expf(-expf(a.pre[(size_t)(tb + tt) * a.H * d + (size_t)head * d + c]));
-            bs[e] = rs[e] * up[c] * ks[e];
+#pragma unroll
+        for (int m = 0; m < RP_FETCH; ++m) {
+            const int e = tid + m * (int)blockDim.x;
+            if (e < nb * d) {
+                const int c = e % d;
+                const float r = ka_to_float(fr[m]), k = ka_to_float(fk[m]);
+                rs[e] = r;
+                ks[e] = k;
+                // (bf16 runs take the hardware's exponential: its error is far below what the projections' rounding leaves)
+                ws[e] = sizeof(T) == 2 ? __expf(-__expf(fw[m])) : expf(-expf(fw[m]));
+                bs[e] = r * up[c] * k;
+            }
+            if (e < nb * dj) vs[e] = ka_to_float(fv[m]);
         }
-        __syncthreads();
-        if (works) {
+        if (tb + TB < t1) fetch(tb + TB);
+        lds_barrier();
+        if constexpr (FAST) {
+            static_assert(!FAST || NI == 4, "the fast form reads four key channels at a time");
+            // A wave has its SIMD to itself, so nothing but its own next loads can hide a load's way through LDS: the
+            // block's tokens are unrolled, token tt + 1's numbers are asked for before token tt's sums, and the partial
+            // read-outs stay in registers until the block is done (a store between the loads would keep them in order).
+            constexpr int RP_BLOCK = 16;                 // (the host gives a block at most this many tokens)
+            if (works) {
+                float outs[RP_BLOCK];
+                float4 r4 = *reinterpret_cast<const float4*>(rs + i0);
+                float4 k4 = *reinterpret_cast<const float4*>(ks + i0);
+                float4 w4 = *reinterpret_cast<const float4*>(ws + i0);
+                float vj = vs[jl];
+#pragma unroll
+                for (int tt = 0; tt < RP_BLOCK; ++tt) {
+                    if (tt < nb) {
+                        float4 rn = r4, kn = k4, wn = w4;
+                        float vn = vj;
+                        if (tt + 1 < nb) {
+                            rn = *reinterpret_cast<const float4*>(rs + (tt + 1) * d + i0);
+                            kn = *reinterpret_cast<const float4*>(ks + (tt + 1) * d + i0);
+                            wn = *reinterpret_cast<const float4*>(ws + (tt + 1) * d + i0);
+                            vn = vs[(tt + 1) * dj + jl];
+                        }
+                        float acc = r4.x * S[0];
+                        S[0] = fmaf(w4.x, S[0], k4.x * vj);
+                        acc = fmaf(r4.y, S[1], acc);
+                        S[1] = fmaf(w4.y, S[1], k4.y * vj);
+                        acc = fmaf(r4.z, S[2], acc);
+                        S[2] = fmaf(w4.z, S[2], k4.z * vj);
+                        acc = fmaf(r4.w, S[3], acc);
+                        S[3] = fmaf(w4.w, S[3], k4.w * vj);
+                        outs[tt] = acc;
+                        r4 = rn; k4 = kn; w4 = wn; vj = vn;
+                    }
+                }
+#pragma unroll
+                for (int tt = 0; tt < RP_BLOCK; ++tt)
+                    if (tt < nb) po[((size_t)tt * P + p) * dj + jl] = outs[tt];
+            }
+        } else if (works) {
             for (int tt = 0; tt < nb; ++tt) {
-                const float vj = vs[tt * d + j];
+                const float vj = vs[tt * dj + jl];
                 const float* r_t = rs + tt * d + i0;
                 const float* k_t = ks + tt * d + i0;
                 const float* w_t = ws + tt * d + i0;
                 float acc = 0.f;
-                if constexpr (FULL) {
 #pragma unroll
-                    for (int ii = 0; ii < NI; ii += 4) {
-                        const float4 r4 = *reinterpret_cast<const float4*>(r_t + ii);
-                        const float4 k4 = *reinterpret_cast<const float4*>(k_t + ii);
-                        const float4 w4 = *reinterpret_cast<const float4*>(w_t + ii);
-                        acc = fmaf(r4.x, S[ii], acc);
-                        S[ii] = fmaf(w4.x, S[ii], k4.x * vj);
-                        acc = fmaf(r4.y, S[ii + 1], acc);
-                        S[ii + 1] = fmaf(w4.y, S[ii + 1], k4.y * vj);
-                        acc = fmaf(r4.z, S[ii + 2], acc);
-                        S[ii + 2] = fmaf(w4.z, S[ii + 2], k4.z * vj);
-                        acc = fmaf(r4.w, S[ii + 3], acc);
-                        S[ii + 3] = fmaf(w4.w, S[ii + 3], k4.w * vj);
-                    }
-                } else {
-#pragma unroll
-                    for (int ii = 0; ii < NI; ++ii) {
-                        if (i0 + ii < d) {
-                            acc = fmaf(r_t[ii], S[ii], acc);
-                            S[ii] = fmaf(w_t[ii], S[ii], k_t[ii] * vj);
-                        }
+                for (int ii = 0; ii < NI; ++ii) {
+                    if (i0 + ii < d) {
+                        acc = fmaf(r_t[ii], S[ii], acc);
+                        S[ii] = fmaf(w_t[ii], S[ii], k_t[ii] * vj);
                     }
                 }
-                po[((size_t)tt * P + p) * d + j] = acc;
+                po[((size_t)tt * P + p) * dj + jl] = acc;
             }
         }
-        __syncthreads();
-        // read-outs of the block: a wave per token, lanes over the value channels
+        lds_barrier();
+        // read-outs of the block: a wave per token; the bonus term's factor is a sum over all key channels, the partial
+        // read-outs are summed per value channel of the slice
         for (int tt = wave; tt < nb; tt += n_waves) {
-            float o[4];
-            float ss = 0.f, bonus = 0.f;
-#pragma unroll
-            for (int q = 0; q < 4; ++q)
-                if (lane + q * KA_WAVE < d) bonus += bs[tt * d + lane + q * KA_WAVE];
+            float bonus = 0.f;
+            for (int c = lane; c < d; c += KA_WAVE) bonus += bs[tt * d + c];
             bonus = ka_wave_sum(bonus);
-#pragma unroll
-            for (int q = 0; q < 4; ++q) {
-                const int c = lane + q * KA_WAVE;
-                o[q] = 0.f;
-                if (c < d) {
-                    float y = bonus * vs[tt * d + c];
-                    for (int pp = 0; pp < P; ++pp) y += po[((size_t)tt * P + pp) * d + c];
-                    o[q] = y;
-                    ss = fmaf(y, y, ss);
-                }
-            }
-            const float inv = 1.0f / sqrtf(ka_wave_sum(ss) / (float)d + a.eps);
-#pragma unroll
-            for (int q = 0; q < 4; ++q) {
-                const int c = lane + q * KA_WAVE;
-                if (c < d) {
-                    const size_t at = (size_t)(tb + tt);
-                    const float g = ka_to_float(gp[at * a.stride + c]);
-                    out[at * a.out_stride + (size_t)head * d + c] = ka_from_float<T>(o[q] * inv * gain[c] * g);
-                }
+            for (int c = lane; c < dj; c += KA_WAVE) {
+                float y = bonus * vs[tt * dj + c];
+                for (int pp = 0; pp < P; ++pp) y += po[((size_t)tt * P + pp) * dj + c];
+                a.raw[(size_t)(tb + tt) * a.H * d + (size_t)head * d + j0 + c] = y;
             }
         }
-        __syncthreads();
+        lds_barrier();
     }
     if (works) {
 #pragma unroll
         for (int ii = 0; ii < NI; ++ii)
             if (i0 + ii < d) S_mem[(size_t)(i0 + ii) * d + j] = S[ii];
     }
-    if (head == 0 && a.x != nullptr) {
+    if (head == 0 && blockIdx.z == 0 && a.x != nullptr) {
         float* kept = a.state + (size_t)slot * a.state_stride + (size_t)a.H * d * d;
         const float* last = a.x + (size_t)(t1 - 1) * a.dim;
         for (int c = tid; c < a.dim; c += blockDim.x) kept[c] = last[c];
     }
 }
 
-// How the kernel cuts a head of d channels: NI state entries a thread, `parts` threads a value channel.
+// out[t, h, :] = raw[t, h, :] / sqrt(mean(raw[t, h, :]^2) + eps) * gain[h, :] * gate[t, h, :]: a wave per (token, head).
+template <typename T>
+__global__ void __launch_bounds__(256)
+decayed_readout_kernel(const float* __restrict__ raw, const float* __restrict__ gain, const T* __restrict__ gate, long gate_stride,
+                       T* __restrict__ out, long out_stride, int n, int H, int d, float eps) {
+    const int pair = blockIdx.x * (blockDim.x / KA_WAVE) + threadIdx.x / KA_WAVE, lane = threadIdx.x % KA_WAVE;
+    if (pair >= n * H) return;
+    const int t = pair / H, head = pair % H;
+    const float* o = raw + (size_t)t * H * d + (size_t)head * d;
+    float ss = 0.f;
+    for (int c = lane; c < d; c += KA_WAVE) ss = fmaf(o[c], o[c], ss);
+    const float inv = 1.0f / sqrtf(ka_wave_sum(ss) / (float)d + eps);
+    for (int c = lane; c < d; c += KA_WAVE)
+        out[(size_t)t * out_stride + (size_t)head * d + c] =
+            ka_from_float<T>(o[c] * inv * gain[(size_t)head * d + c] * ka_to_float(gate[(size_t)t * gate_stride + (size_t)head * d + c]));
+}
+
+// How the general form cuts a head of d channels: NI state entries a thread, `parts` threads a value channel.
 static bool decay_shape(int d, int* ni, int* parts) {
     if (d <= 0 || d > 256) return false;
-    for (int cand : {4, 8, 16, 32, 64}) {
+    for (int cand : {16, 32, 64}) {
         const int pp = (d + cand - 1) / cand;
-        if ((long)pp * d <= 1024) {
+        if ((long)pp * d <= (cand == 64 ? 1024 : 512)) {
             *ni = cand;
             *parts = pp;
             return true;
@@ -228,34 +287,52 @@ KA_API int ka_decayed_memory_supported(int d) {
     return decay_shape(d, &ni, &parts) ? 1 : 0;
 }
 
+// raw: fp32 scratch [n, H d] of the caller's.
 KA_API int ka_decayed_memory(const void* r, const void* k, const void* v, const void* gate, long stride, int dtype, const float* pre,
                              const float* u, const float* gain, float* state, long state_stride, const float* x, int dim,
-                             const int* cu_q, const int* row_slot, void* out, long out_stride, int n_rows, int H, int d, float eps,
-                             hipStream_t stream) {
+                             const int* cu_q, const int* row_slot, void* out, long out_stride, int n, int n_rows, int H, int d, float eps,
+                             float* raw, hipStream_t stream) {
     const char* who = "ka_decayed_memory";
-    KA_CHECK(n_rows >= 0 && H > 0 && d > 0 && eps >= 0.f, "%s: bad sizes", who);
+    KA_CHECK(n >= 0 && n_rows >= 0 && H > 0 && d > 0 && eps >= 0.f && raw != nullptr, "%s: bad sizes", who);
     KA_CHECK(dtype == KA_F32 || dtype == KA_BF16, "%s: unsupported dtype %d", who, dtype);
     int ni = 0, parts = 0;
     KA_CHECK(decay_shape(d, &ni, &parts), "%s: heads of %d channels are not covered (up to 256)", who, d);
     KA_CHECK(state_stride >= (long)H * d * d + (x ? dim : 0), "%s: the state rows are too short", who);
     KA_CHECK(H <= 65535 && n_rows <= 65535, "%s: too many heads or rows", who);
-    if (n_rows == 0) return 0;
-    int block_tokens = 49152 / (d * 4 * (5 + parts));
-    block_tokens = block_tokens < 1 ? 1 : (block_tokens > 16 ? 16 : block_tokens);
-    const int threads = ((parts * d + KA_WAVE - 1) / KA_WAVE) * KA_WAVE;
-    const size_t lds = (size_t)block_tokens * d * (5 + parts) * sizeof(float);
-    const bool full = d % ni == 0 && d % 4 == 0;
-    DecayArgs a{r, k, v, gate, stride, pre, u, gain, state, state_stride, x, dim, cu_q, row_slot, out, out_stride, H, d, block_tokens, parts, eps};
-    dim3 grid(H, n_rows);
-#define RP_LAUNCH(T, NI)                                                                                             \
-    if (ni == NI) {                                                                                                  \
-        if (full) hipLaunchKernelGGL((decayed_memory_kernel<T, NI, true>), grid, dim3(threads), lds, stream, a);     \
-        else hipLaunchKernelGGL((decayed_memory_kernel<T, NI, false>), grid, dim3(threads), lds, stream, a);         \
+    if (n_rows == 0 || n == 0) return 0;
+    const bool fast = d % RP_SLICE == 0;
+    int slice = d, fetch = ni == 64 ? 2 : 8;
+    if (fast) {
+        ni = 4;
+        parts = d / 4;
+        slice = d > 128 ? RP_SLICE / 2 : RP_SLICE;          // (at most 512 threads a workgroup)
+        fetch = 4;
     }
-#define RP_LAUNCH_ALL(T) RP_LAUNCH(T, 4) RP_LAUNCH(T, 8) RP_LAUNCH(T, 16) RP_LAUNCH(T, 32) RP_LAUNCH(T, 64)
+    const int threads = ((parts * slice + KA_WAVE - 1) / KA_WAVE) * KA_WAVE;
+    int block_tokens = 49152 / (4 * (4 * d + slice * (1 + parts)));
+    block_tokens = block_tokens < 1 ? 1 : (block_tokens > 16 ? 16 : block_tokens);
+    if (block_tokens > fetch * threads / d) block_tokens = fetch * threads / d;          // (what a thread fetches of a block)
+    if (block_tokens < 1) block_tokens = 1;
+    const size_t lds = (size_t)block_tokens * (4 * d + slice * (1 + parts)) * sizeof(float);
+    DecayArgs a{r, k, v, stride, pre, u, state, state_stride, x, dim, cu_q, row_slot, raw, H, d, block_tokens, parts, slice};
+    dim3 grid(H, n_rows, d / slice);
+#define RP_LAUNCH(T, NI, FAST) hipLaunchKernelGGL((decayed_memory_kernel<T, NI, FAST>), grid, dim3(threads), lds, stream, a)
+#define RP_LAUNCH_ALL(T)                                                            \
+    if (fast) RP_LAUNCH(T, 4, true);                                                \
+    else if (ni == 16) RP_LAUNCH(T, 16, false);                                     \
+    else if (ni == 32) RP_LAUNCH(T, 32, false);                                     \
+    else RP_LAUNCH(T, 64, false);
     if (dtype == KA_F32) { RP_LAUNCH_ALL(float) } else { RP_LAUNCH_ALL(bf16_t) }
 #undef RP_LAUNCH_ALL
 #undef RP_LAUNCH
+    KA_LAUNCH_CHECK();
+    const int pairs = n * H;
+    if (dtype == KA_F32)
+        hipLaunchKernelGGL(decayed_readout_kernel<float>, dim3((pairs + 3) / 4), dim3(256), 0, stream, raw, gain, (const float*)gate, stride,
+                           (float*)out, out_stride, n, H, d, eps);
+    else
+        hipLaunchKernelGGL(decayed_readout_kernel<bf16_t>, dim3((pairs + 3) / 4), dim3(256), 0, stream, raw, gain, (const bf16_t*)gate, stride,
+                           (bf16_t*)out, out_stride, n, H, d, eps);
     KA_LAUNCH_CHECK();
     return 0;
 }

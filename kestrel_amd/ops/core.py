@@ -59,8 +59,8 @@ _SIGNATURES = {
     "ka_token_shift": [_c_void_p, _c_void_p, _c_long, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int,
                        _c_int, _c_void_p],
     "ka_decayed_memory": [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_long, _c_int, _c_void_p, _c_void_p, _c_void_p, _c_void_p,
-                          _c_long, _c_void_p, _c_int, _c_void_p, _c_void_p, _c_void_p, _c_long, _c_int, _c_int, _c_int, _c_float,
-                          _c_void_p],
+                          _c_long, _c_void_p, _c_int, _c_void_p, _c_void_p, _c_void_p, _c_long, _c_int, _c_int, _c_int, _c_int, _c_float,
+                          _c_void_p, _c_void_p],
     "ka_route": [_c_void_p, _c_long, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_void_p, _c_void_p, _c_void_p],
     "ka_experts_linear": [_c_void_p, _c_long, _c_int, _c_void_p, _c_int, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void_p,
                           _c_long, _c_int, _c_void_p],
@@ -679,13 +679,14 @@ def decayed_memory_supported(head_dim: int) -> bool:
 
 def decayed_memory(r: torch.Tensor, k: torch.Tensor, v: torch.Tensor, gate: torch.Tensor, pre: torch.Tensor, u: torch.Tensor,
                    gain: torch.Tensor, state: torch.Tensor, x: Optional[torch.Tensor], cu_q: torch.Tensor, row_slot: torch.Tensor,
-                   out: torch.Tensor, n_heads: int, head_dim: int, eps: float) -> None:
+                   out: torch.Tensor, n_heads: int, head_dim: int, eps: float, raw: Optional[torch.Tensor] = None) -> None:
     """A decaying matrix memory over the packed tokens of a step. Per head a state ``S`` ``[d, d]``; for every token of a row, in
     order: ``o_j = sum_i r_i (S_ij + u_i k_i v_j)``, then ``S_ij <- exp(-exp(pre_i)) S_ij + k_i v_j``; ``o`` divided by its root mean
     square over the head (``eps``), times ``gain``, times ``gate``. ``r, k, v, gate``: ``[n, H d]`` views of one type with one
     row stride; ``pre`` fp32 ``[n, H d]``; ``u``, ``gain`` fp32 ``[H d]``; ``state`` fp32 ``[slots + 1, H d d + dim]``, a row per
     request slot: the matrices, then the stream's last row (``x`` fp32 ``[n, dim]``, kept for the next step's token shift;
-    ``None``: the rows hold the matrices alone). A row of the step without a request writes zeros and touches no state."""
+    ``None``: the rows hold the matrices alone). A row of the step without a request writes zeros and touches no state.
+    ``raw``: fp32 scratch ``[n, H d]`` for the read-outs before their norm (a captured step passes its workspace's)."""
     _dev(r, k, v, gate, pre, u, gain, state, x, cu_q, row_slot, out)
     n = r.shape[0]
     width = n_heads * head_dim
@@ -702,10 +703,13 @@ def decayed_memory(r: torch.Tensor, k: torch.Tensor, v: torch.Tensor, gate: torc
     n_rows = row_slot.numel()
     _need(cu_q.dtype == torch.int32 and cu_q.numel() == n_rows + 1 and row_slot.dtype == torch.int32, "decayed_memory: cu_q int32 [rows + 1]")
     _need(out.dtype == r.dtype and out.dim() == 2 and out.stride(1) == 1 and tuple(out.shape) == (n, width), "decayed_memory: out [n, H d]")
+    if raw is None:
+        raw = torch.empty((n, width), dtype=torch.float32, device=r.device)
+    _need(raw.dtype == torch.float32 and raw.is_contiguous() and raw.numel() >= n * width and raw.is_cuda, "decayed_memory: raw fp32 [n, H d]")
     _check(lib().ka_decayed_memory(r.data_ptr(), k.data_ptr(), v.data_ptr(), gate.data_ptr(), r.stride(0) if n > 1 else width,
                                    code_of(r.dtype), pre.data_ptr(), u.data_ptr(), gain.data_ptr(), state.data_ptr(), state.stride(0),
                                    _ptr(x), dim, cu_q.data_ptr(), row_slot.data_ptr(), out.data_ptr(),
-                                   out.stride(0) if n > 1 else width, n_rows, n_heads, head_dim, float(eps), stream_ptr()))
+                                   out.stride(0) if n > 1 else width, n, n_rows, n_heads, head_dim, float(eps), raw.data_ptr(), stream_ptr()))
 
 
 def route(logits: torch.Tensor, n_outputs: int, correction: Optional[torch.Tensor], top: int, n_groups: int, keep_groups: int,

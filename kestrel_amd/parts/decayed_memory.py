@@ -32,7 +32,7 @@ class DecayedMemory(Mixer):
     The mixer reads the fp32 stream itself (``reads_stream``): the mixes are computed in fp32 and rounded once to the
     activation type. The five projections are linears of that type; the second linear of the decay writes fp32 (with
     ``w0`` as its bias) and the exponentials are taken in the recurrence kernel, so that everything that enters the
-    recurrence besides the projections is fp32. One kernel walks over every row's tokens in order
+    recurrence besides the projections is fp32. One kernel walks over every row's tokens in order and a second normalises the read-outs
     (``ops.core.decayed_memory``), whatever the step holds: a prompt, a portion, single tokens. Rows without a request
     (the padding of a replayed step) write zeros and touch no state."""
 
@@ -99,8 +99,9 @@ class DecayedMemory(Mixer):
         linear(low, self.w_2, self.w_0, pre)
         out = ws.get("decay.out", (n, self.width), self.dtype)
         r, k, v, g = (rkvg[:, i * self.width:(i + 1) * self.width] for i in range(4))
+        raw = ws.get("decay.raw", (n, self.width), torch.float32)
         core.decayed_memory(r, k, v, g, pre, self.u, self.gain, state, x, batch.cu_q, batch.row_slot, out, spec.n_heads,
-                            spec.head_dim, spec.eps)
+                            spec.head_dim, spec.eps, raw=raw)
         return out
 
     def output_projection(self):
