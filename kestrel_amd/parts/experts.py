@@ -23,12 +23,12 @@ class RoutedExperts(FeedForward):
 
     When the weights are bound, the experts' ``gate`` and ``up`` rows are laid in pairs and the experts stacked
     (``[E, 2 hidden, dim]``, ``[E, dim, hidden]``). A step runs: the router's linear (fp32), the choice
-    (``ops.core.route``), the experts' two linears, and the weighted sum. In bf16 steps with at least
-    ``PAIRS_BY_EXPERT_FROM`` pairs and two pairs an expert on average, the pairs are listed by expert and each expert's
-    pairs go through the matrix cores together (``ops.fast.experts_feed_forward_bf16``); otherwise, and in fp32, every pair
-    is computed by itself, its expert's weights streamed once for it (``ops.core.experts_linear``: with fewer pairs than
-    experts that reads no more than the list would, at twice the rate: 3.6 against 1.9 TB/s at 48 pairs over 62 experts).
-    Either way a pair's result depends on its own row alone."""
+    (``ops.core.route``), the experts' two linears, and the weighted sum. In bf16 steps of at least
+    ``PAIRS_BY_EXPERT_FROM`` pairs, the pairs are listed by expert and each expert's pairs go through the matrix cores
+    together (``ops.fast.experts_feed_forward_bf16``); otherwise, and in fp32, every pair is computed by itself, its expert's
+    weights streamed once for it (``ops.core.experts_linear``). Measured at 48 pairs over 62 experts, where the lists hold
+    hardly more than a pair an expert: 1.28 ms a step by lists, 1.42 pair by pair. Either way a pair's result depends on
+    its own row alone."""
 
     replays_every_step = True
     PAIRS_BY_EXPERT_FROM = 33
@@ -101,7 +101,7 @@ class RoutedExperts(FeedForward):
         hidden = ws.get("experts.hidden", (n * top, spec.hidden_dim), self.dtype)
         y = ws.get("experts.y", (n * top, spec.dim), torch.float32)
         done = False
-        if self.dtype == torch.bfloat16 and n * top >= max(self.PAIRS_BY_EXPERT_FROM, 2 * E):
+        if self.dtype == torch.bfloat16 and n * top >= self.PAIRS_BY_EXPERT_FROM:
             from ..ops import fast
             done = fast.experts_feed_forward_bf16(h, self.pairs, self.down, chosen, hidden, y, self.act, ws)
         if not done:
