@@ -73,7 +73,7 @@ route_kernel(const float* __restrict__ logits, long stride, const float* __restr
             allowed_s[lane] = 0;
         }
         __syncthreads();
-        for (int round = 0; round < keep; ++round) {
+        for (int turn = 0; turn < keep; ++turn) {
             float v = lane < n_groups && !allowed_s[lane] ? group_s[lane] : -INFINITY;
             int i = lane < n_groups && !allowed_s[lane] ? lane : 0x7fffffff;
             ex_wave_argmax(v, i);
