@@ -126,19 +126,29 @@ __global__ void __launch_bounds__(!FAST && NI == 64 ? 1024 : 512) decayed_memory
     constexpr int RP_FETCH = FAST ? 4 : (NI == 64 ? 2 : 8);      // (the host sizes the block so that a thread has at most this many)
     T fr[RP_FETCH], fk[RP_FETCH], fv[RP_FETCH];
     float fw[RP_FETCH];
+    // (which token of a block and which channel an element is does not change from block to block: the divisions are done once)
+    int e_tok[RP_FETCH], e_ch[RP_FETCH], v_tok[RP_FETCH], v_ch[RP_FETCH];
+    float e_u[RP_FETCH];
+#pragma unroll
+    for (int m = 0; m < RP_FETCH; ++m) {
+        const int e = tid + m * (int)blockDim.x;
+        e_tok[m] = e / d;
+        e_ch[m] = e % d;
+        v_tok[m] = e / dj;
+        v_ch[m] = e % dj;
+        e_u[m] = up[e_ch[m]];
+    }
     auto fetch = [&](int tb) {
         const int nb = min(TB, t1 - tb);
 #pragma unroll
         for (int m = 0; m < RP_FETCH; ++m) {
-            const int e = tid + m * (int)blockDim.x;
-            if (e < nb * d) {
-                const int tt = e / d, c = e % d;
-                const size_t at = (size_t)(tb + tt) * a.stride + c;
+            if (e_tok[m] < nb) {
+                const size_t at = (size_t)(tb + e_tok[m]) * a.stride + e_ch[m];
                 fr[m] = rp[at];
                 fk[m] = kp[at];
-                fw[m] = a.pre[(size_t)(tb + tt) * a.H * d + (size_t)head * d + c];
+                fw[m] = a.pre[(size_t)(tb + e_tok[m]) * a.H * d + (size_t)head * d + e_ch[m]];
             }
-            if (e < nb * dj) fv[m] = vp[(size_t)(tb + e / dj) * a.stride + j0 + e % dj];
+            if (v_tok[m] < nb) fv[m] = vp[(size_t)(tb + v_tok[m]) * a.stride + j0 + v_ch[m]];
         }
     };
     // This wave's LDS writes done, then everybody's: what __syncthreads() does too, but that one also waits for every load
@@ -155,16 +165,15 @@ __global__ void __launch_bounds__(!FAST && NI == 64 ? 1024 : 512) decayed_memory
 #pragma unroll
         for (int m = 0; m < RP_FETCH; ++m) {
             const int e = tid + m * (int)blockDim.x;
-            if (e < nb * d) {
-                const int c = e % d;
+            if (e_tok[m] < nb) {
                 const float r = ka_to_float(fr[m]), k = ka_to_float(fk[m]);
                 rs[e] = r;
                 ks[e] = k;
                 // (bf16 runs take the hardware's exponential: its error is far below what the projections' rounding leaves)
                 ws[e] = sizeof(T) == 2 ? __expf(-__expf(fw[m])) : expf(-expf(fw[m]));
-                bs[e] = r * up[c] * k;
+                bs[e] = r * e_u[m] * k;
             }
-            if (e < nb * dj) vs[e] = ka_to_float(fv[m]);
+            if (v_tok[m] < nb) vs[e] = ka_to_float(fv[m]);
         }
         if (tb + TB < t1) fetch(tb + TB);
         lds_barrier();
@@ -176,20 +185,30 @@ __global__ void __launch_bounds__(!FAST && NI == 64 ? 1024 : 512) decayed_memory
             constexpr int RP_BLOCK = 16;                 // (the host gives a block at most this many tokens)
             if (works) {
                 float outs[RP_BLOCK];
-                float4 r4 = *reinterpret_cast<const float4*>(rs + i0);
-                float4 k4 = *reinterpret_cast<const float4*>(ks + i0);
-                float4 w4 = *reinterpret_cast<const float4*>(ws + i0);
-                float vj = vs[jl];
+                // (four tokens ahead: a trip through LDS, with the workgroup's other waves asking too, takes as long as three
+                // or four tokens' sums)
+                constexpr int RP_AHEAD = 4;
+                float4 rq[RP_AHEAD], kq[RP_AHEAD], wq[RP_AHEAD];
+                float vq[RP_AHEAD];
+#pragma unroll
+                for (int q = 0; q < RP_AHEAD; ++q) {
+                    if (q < nb) {
+                        rq[q] = *reinterpret_cast<const float4*>(rs + q * d + i0);
+                        kq[q] = *reinterpret_cast<const float4*>(ks + q * d + i0);
+                        wq[q] = *reinterpret_cast<const float4*>(ws + q * d + i0);
+                        vq[q] = vs[q * dj + jl];
+                    }
+                }
 #pragma unroll
                 for (int tt = 0; tt < RP_BLOCK; ++tt) {
                     if (tt < nb) {
-                        float4 rn = r4, kn = k4, wn = w4;
-                        float vn = vj;
-                        if (tt + 1 < nb) {
-                            rn = *reinterpret_cast<const float4*>(rs + (tt + 1) * d + i0);
-                            kn = *reinterpret_cast<const float4*>(ks + (tt + 1) * d + i0);
-                            wn = *reinterpret_cast<const float4*>(ws + (tt + 1) * d + i0);
-                            vn = vs[(tt + 1) * dj + jl];
+                        const float4 r4 = rq[tt % RP_AHEAD], k4 = kq[tt % RP_AHEAD], w4 = wq[tt % RP_AHEAD];
+                        const float vj = vq[tt % RP_AHEAD];
+                        if (tt + RP_AHEAD < nb) {
+                            rq[tt % RP_AHEAD] = *reinterpret_cast<const float4*>(rs + (tt + RP_AHEAD) * d + i0);
+                            kq[tt % RP_AHEAD] = *reinterpret_cast<const float4*>(ks + (tt + RP_AHEAD) * d + i0);
+                            wq[tt % RP_AHEAD] = *reinterpret_cast<const float4*>(ws + (tt + RP_AHEAD) * d + i0);
+                            vq[tt % RP_AHEAD] = vs[(tt + RP_AHEAD) * dj + jl];
                         }
                         float acc = r4.x * S[0];
                         S[0] = fmaf(w4.x, S[0], k4.x * vj);
@@ -200,12 +219,27 @@ __global__ void __launch_bounds__(!FAST && NI == 64 ? 1024 : 512) decayed_memory
                         acc = fmaf(r4.w, S[3], acc);
                         S[3] = fmaf(w4.w, S[3], k4.w * vj);
                         outs[tt] = acc;
-                        r4 = rn; k4 = kn; w4 = wn; vj = vn;
                     }
                 }
+                // With 16 value channels a workgroup a wave holds four parts of every channel, 16 lanes apart: they meet
+                // inside the wave (two swaps of rows and halves), and one lane in four writes.
+                const bool meet = dj == 16;
 #pragma unroll
-                for (int tt = 0; tt < RP_BLOCK; ++tt)
-                    if (tt < nb) po[((size_t)tt * P + p) * dj + jl] = outs[tt];
+                for (int tt = 0; tt < RP_BLOCK; ++tt) {
+                    if (tt < nb) {
+                        float y = outs[tt];
+                        if (meet) {
+                            float y1, y2;
+                            ka_lanes_pair<16>(y, y1, y2);
+                            y = y1 + y2;
+                            ka_lanes_pair<32>(y, y1, y2);
+                            y = y1 + y2;
+                            if (lane < 16) po[((size_t)tt * P + wave * 4) * dj + jl] = y;
+                        } else {
+                            po[((size_t)tt * P + p) * dj + jl] = y;
+                        }
+                    }
+                }
             }
         } else if (works) {
             for (int tt = 0; tt < nb; ++tt) {
@@ -227,13 +261,29 @@ __global__ void __launch_bounds__(!FAST && NI == 64 ? 1024 : 512) decayed_memory
         lds_barrier();
         // read-outs of the block: a wave per token; the bonus term's factor is a sum over all key channels, the partial
         // read-outs are summed per value channel of the slice
+        if (FAST && dj == 16 && (int)blockDim.x >= TB * 16) {
+            // an output a thread: token tid / 16, channel tid % 16; the 16 lanes of a token sum u r k over the key channels
+            // between them (a row of the vector unit's lane moves)
+            const int tt = tid / 16, c = tid % 16;
+            float part = 0.f;
+            if (tt < nb)
+                for (int q = c; q < d; q += 16) part += bs[tt * d + q];
+            const float bonus = ka_lanes_reduce<1, 16>(part, KaSum{});
+            if (tt < nb) {
+                float y = bonus * vs[tt * dj + c];
+                for (int pp = 0; pp < P; pp += 4) y += po[((size_t)tt * P + pp) * dj + c];
+                a.raw[(size_t)(tb + tt) * a.H * d + (size_t)head * d + j0 + c] = y;
+            }
+        } else
         for (int tt = wave; tt < nb; tt += n_waves) {
             float bonus = 0.f;
             for (int c = lane; c < d; c += KA_WAVE) bonus += bs[tt * d + c];
             bonus = ka_wave_sum(bonus);
             for (int c = lane; c < dj; c += KA_WAVE) {
                 float y = bonus * vs[tt * dj + c];
-                for (int pp = 0; pp < P; ++pp) y += po[((size_t)tt * P + pp) * dj + c];
+                // (the fast form with 16 channels a workgroup has left one sum a wave, at the place of the wave's first part)
+                const int hop = FAST && dj == 16 ? 4 : 1;
+                for (int pp = 0; pp < P; pp += hop) y += po[((size_t)tt * P + pp) * dj + c];
                 a.raw[(size_t)(tb + tt) * a.H * d + (size_t)head * d + j0 + c] = y;
             }
         }
