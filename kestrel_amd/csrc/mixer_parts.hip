@@ -388,11 +388,14 @@ KA_API int ka_gated_pairs(const void* x, long x_stride, void* out, long out_stri
 
 // ----------------------------------------------------------------------------
 // The sum of normalised branches into the stream: x += ca * rms(a) * gain_a [+ cb * rms(b) * gain_b], every
-// branch divided by its own root mean square over the row; all fp32.
+// branch divided by its own root mean square over the row; all fp32. `rounded` (optional, of type TR): the new rows of the
+// stream are left there as well, in the activation type, for a reader that takes them so.
 // ----------------------------------------------------------------------------
+template <typename TR>
 __global__ void __launch_bounds__(MP_THREADS)
 branches_sum_kernel(float* __restrict__ x, const float* __restrict__ a, const float* __restrict__ gain_a, float ca,
-                    const float* __restrict__ b, const float* __restrict__ gain_b, float cb, float eps, int dim) {
+                    const float* __restrict__ b, const float* __restrict__ gain_b, float cb, float eps, int dim,
+                    TR* __restrict__ rounded) {
     __shared__ float smem[MP_WAVES];
     const size_t at = (size_t)blockIdx.x * dim;
     float sa = 0.f, sb = 0.f;
@@ -405,15 +408,23 @@ branches_sum_kernel(float* __restrict__ x, const float* __restrict__ a, const fl
     for (int d = threadIdx.x; d < dim; d += MP_THREADS) {
         float y = ca * (a[at + d] * ra * (gain_a ? gain_a[d] : 1.f));
         if (b) y += cb * (b[at + d] * rb * (gain_b ? gain_b[d] : 1.f));
-        x[at + d] += y;
+        y += x[at + d];
+        x[at + d] = y;
+        if (rounded) rounded[at + d] = ka_from_float<TR>(y);
     }
 }
 
 KA_API int ka_branches_sum(float* x, const float* a, const float* gain_a, float ca, const float* b, const float* gain_b,
-                           float cb, float eps, int n, int dim, hipStream_t stream) {
+                           float cb, float eps, int n, int dim, void* rounded, int rounded_dtype, hipStream_t stream) {
     KA_CHECK(n >= 0 && dim > 0 && eps >= 0.f && a != nullptr, "ka_branches_sum: bad sizes");
+    KA_CHECK(rounded == nullptr || rounded_dtype == KA_F32 || rounded_dtype == KA_BF16, "ka_branches_sum: unsupported dtype %d", rounded_dtype);
     if (n == 0) return 0;
-    hipLaunchKernelGGL(branches_sum_kernel, dim3(n), dim3(MP_THREADS), 0, stream, x, a, gain_a, ca, b, gain_b, cb, eps, dim);
+    if (rounded != nullptr && rounded_dtype == KA_BF16)
+        hipLaunchKernelGGL(branches_sum_kernel<bf16_t>, dim3(n), dim3(MP_THREADS), 0, stream, x, a, gain_a, ca, b, gain_b, cb, eps, dim,
+                           (bf16_t*)rounded);
+    else
+        hipLaunchKernelGGL(branches_sum_kernel<float>, dim3(n), dim3(MP_THREADS), 0, stream, x, a, gain_a, ca, b, gain_b, cb, eps, dim,
+                           (float*)rounded);
     KA_LAUNCH_CHECK();
     return 0;
 }

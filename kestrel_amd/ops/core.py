@@ -52,7 +52,7 @@ _SIGNATURES = {
     "ka_add_vector": [_c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_void_p],
     "ka_gate_mul": [_c_void_p, _c_long, _c_void_p, _c_long, _c_int, _c_int, _c_int, _c_void_p],
     "ka_branches_sum": [_c_void_p, _c_void_p, _c_void_p, _c_float, _c_void_p, _c_void_p, _c_float, _c_float, _c_int, _c_int,
-                        _c_void_p],
+                        _c_void_p, _c_int, _c_void_p],
     "ka_matrix_memory": [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_long, _c_int, _c_void_p, _c_void_p, _c_int, _c_void_p,
                          _c_void_p, _c_void_p, _c_void_p, _c_long, _c_int, _c_int, _c_int, _c_int, _c_float, _c_float, _c_float,
                          _c_int, _c_void_p],
@@ -597,17 +597,20 @@ def gate_mul(x: torch.Tensor, gate: torch.Tensor) -> None:
 
 
 def branches_sum(x: torch.Tensor, a: torch.Tensor, gain_a: Optional[torch.Tensor], weight_a: float,
-                 b: Optional[torch.Tensor] = None, gain_b: Optional[torch.Tensor] = None, weight_b: float = 0.0, eps: float = 0.0) -> None:
+                 b: Optional[torch.Tensor] = None, gain_b: Optional[torch.Tensor] = None, weight_b: float = 0.0, eps: float = 0.0,
+                 rounded: Optional[torch.Tensor] = None) -> None:
     """``x += weight_a * rms(a) * gain_a + weight_b * rms(b) * gain_b``: every branch divided by its own root mean square
-    ``sqrt(mean(square) + eps)`` over the row; all contiguous fp32 ``[n, dim]``, gains fp32 ``[dim]``."""
-    _dev(x, a, gain_a, b, gain_b)
+    ``sqrt(mean(square) + eps)`` over the row; all contiguous fp32 ``[n, dim]``, gains fp32 ``[dim]``. ``rounded`` (contiguous
+    ``[n, dim]`` of either type): the new rows of ``x`` are written there as well."""
+    _dev(x, a, gain_a, b, gain_b, rounded)
     n, dim = x.shape
     for t in (x, a, b):
         _need(t is None or (t.dtype == torch.float32 and t.is_contiguous() and tuple(t.shape) == (n, dim)), "branches_sum: contiguous fp32 [n, dim]")
     for g in (gain_a, gain_b):
         _need(g is None or (g.dtype == torch.float32 and g.numel() == dim and g.is_contiguous()), "branches_sum: gains fp32 [dim]")
+    _need(rounded is None or (rounded.is_contiguous() and tuple(rounded.shape) == (n, dim)), "branches_sum: rounded must be contiguous [n, dim]")
     _check(lib().ka_branches_sum(x.data_ptr(), a.data_ptr(), _ptr(gain_a), float(weight_a), _ptr(b), _ptr(gain_b), float(weight_b),
-                                 float(eps), n, dim, stream_ptr()))
+                                 float(eps), n, dim, _ptr(rounded), code_of(rounded.dtype) if rounded is not None else 0, stream_ptr()))
 
 
 def matrix_memory(projected: torch.Tensor, offsets, pre: torch.Tensor, state: torch.Tensor, cu_q: torch.Tensor,

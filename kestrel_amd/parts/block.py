@@ -253,13 +253,19 @@ def _output_norms(block: "Block", x, batch, cache) -> None:
         core.cast_columns(x, h)
         return h
 
-    def add(norm) -> None:
+    def add(norm, also_rounded: bool = False) -> bool:
+        """``x += norm(delta)``; with ``also_rounded`` the stream's rounding is left in ``block.h`` by the same launch where
+        the norm offers that (returns whether it did)."""
         if callable(getattr(norm, "add_normed", None)):
+            if also_rounded and block.dtype != torch.float32:
+                norm.add_normed(delta, x, rounded=ws.get("block.h", tuple(x.shape), block.dtype))
+                return True
             norm.add_normed(delta, x)
-        else:
-            normed = ws.get("block.normed", tuple(x.shape), torch.float32)
-            norm.forward(delta, normed)
-            core.add_scaled(x, normed, 1.0)
+            return False
+        normed = ws.get("block.normed", tuple(x.shape), torch.float32)
+        norm.forward(delta, normed)
+        core.add_scaled(x, normed, 1.0)
+        return False
 
     mixer = block.mixer
     source = x if getattr(mixer, "reads_stream", False) else rounded()
@@ -268,10 +274,11 @@ def _output_norms(block: "Block", x, batch, cache) -> None:
     else:
         delta.zero_()
         mixer.forward(source, batch, cache, delta)
-    add(block.norm)
     ff = block.feed_forward
+    left = add(block.norm, also_rounded=ff is not None)
     if ff is not None:
-        h = rounded()
+        # (the feed-forward reads the stream's rounding, which the launch before has left where the norm could)
+        h = ws.get("block.h", tuple(x.shape), block.dtype) if left else rounded()
         if callable(getattr(ff, "mix", None)):
             ff.mix(h, batch, delta, False)
         else:

@@ -65,9 +65,10 @@ class RMSNorm(Norm):
     def forward(self, x, out, rows=None) -> None:
         core.rmsnorm(x, self.weight, self.spec.eps, out, rows)
 
-    def add_normed(self, y, x) -> None:
-        """``x += norm(y)`` for fp32 rows ``y`` into the fp32 stream ``x`` (a norm that stands behind a sublayer)."""
-        core.branches_sum(x, y, self.weight, 1.0, eps=float(self.spec.eps))
+    def add_normed(self, y, x, rounded=None) -> None:
+        """``x += norm(y)`` for fp32 rows ``y`` into the fp32 stream ``x`` (a norm that stands behind a sublayer); ``rounded``:
+        the new rows of the stream are left there too, in that tensor's type."""
+        core.branches_sum(x, y, self.weight, 1.0, eps=float(self.spec.eps), rounded=rounded)
 
     def rms_operands(self):
         """``(weight fp32 [dim], eps)`` of ``x / sqrt(mean(x^2) + eps) * weight``."""
