@@ -178,7 +178,8 @@ __global__ void __launch_bounds__(MP_THREADS) qkv_prepare_kernel(PrepareArgs a) 
 
 // The same for bf16 rows whose heads are 32, 64 or 128 channels wide: a lane takes eight neighbouring channels with one
 // 16-byte load, LPH lanes a head, so that a wave covers 64 / LPH heads at a time and a head's sum of squares meets inside
-// its lanes. A rotated pair (channels 2i and 2i + 1 only) lies inside a lane's eight. Values in pieces of eight as well.
+// its lanes. A rotated pair of neighbours (channels 2i and 2i + 1) lies inside a lane's eight; a pair of halves (i and
+// i + rot / 2, rot a multiple of 16) in two lanes of the head, which exchange their numbers. Values in pieces of eight as well.
 typedef __attribute__((ext_vector_type(8))) __bf16 mp_bf16x8;
 typedef __attribute__((ext_vector_type(4))) float mp_floatx4;
 
@@ -249,7 +250,7 @@ __global__ void __launch_bounds__(MP_THREADS) qkv_prepare_wide_kernel(PrepareArg
 #pragma unroll
             for (int u = 0; u < 4; ++u) { y[u] *= g0[u]; y[4 + u] *= g1[u]; }
         }
-        if (a.freqs) {
+        if (a.freqs && a.interleaved) {
 #pragma unroll
             for (int p = 0; p < 4; ++p) {
                 const int i = sub * 4 + p;
@@ -257,6 +258,22 @@ __global__ void __launch_bounds__(MP_THREADS) qkv_prepare_wide_kernel(PrepareArg
                     const float u = y[2 * p], v = y[2 * p + 1];
                     y[2 * p] = u * cs[i] - v * sn[i];
                     y[2 * p + 1] = v * cs[i] + u * sn[i];
+                }
+            }
+        } else if (a.freqs) {
+            // halves: channel c turns with channel c + rot / 2, which the lane rot / 16 further on holds (rot is a multiple
+            // of 16 here): the lanes of a pair exchange their eight numbers
+            const int apart = a.rot / 16;
+            const bool low = sub < apart, turned = sub < 2 * apart;
+            const int partner = (tid % KA_WAVE) + (low ? apart : -apart);
+            float other[8];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) other[u] = __shfl(y[u], turned ? partner : tid % KA_WAVE);
+            if (turned) {
+#pragma unroll
+                for (int u = 0; u < 8; ++u) {
+                    const int i = (low ? sub : sub - apart) * 8 + u;
+                    y[u] = low ? y[u] * cs[i] - other[u] * sn[i] : y[u] * cs[i] + other[u] * sn[i];
                 }
             }
         }
@@ -315,7 +332,7 @@ KA_API int ka_qkv_prepare(void* qkv, int dtype, long row_stride, const int* posi
                   freqs, rot, interleaved, q_coef, q_every, blend, v_other, v_other_stride, lambda, v_from_k};
     // bf16 heads of 32, 64 or 128 channels, everything 16-byte aligned, pairs of neighbours if rotated: eight channels a lane
     const bool wide = dtype == KA_BF16 && (hd == 32 || hd == 64 || hd == 128) && hdv % 8 == 0 && row_stride % 8 == 0 &&
-        (uintptr_t)qkv % 16 == 0 && (freqs == nullptr || interleaved == 1) &&
+        (uintptr_t)qkv % 16 == 0 && (freqs == nullptr || interleaved == 1 || rot % 16 == 0) &&
         (blend == 0 || ((uintptr_t)v_other % 16 == 0 && v_other_stride % 8 == 0)) &&
         (uintptr_t)q_gain % 16 == 0 && (uintptr_t)k_gain % 16 == 0 && (slots == nullptr || (uintptr_t)k_cache % 16 == 0);
     if (wide && hd == 32) hipLaunchKernelGGL(qkv_prepare_wide_kernel<4>, dim3(n), dim3(MP_THREADS), lds, stream, a);

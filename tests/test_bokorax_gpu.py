@@ -325,13 +325,15 @@ def test_capped_scores_sinks_per_head_and_a_gate_per_head(kernel, dtype, heads, 
 
 
 @pytest.mark.parametrize("dtype", DTYPES, ids=DTYPE_IDS)
-def test_prepare_kernel_values_from_keys_and_queries_alone(dtype):
+@pytest.mark.parametrize("d, rot", [(24, 12), (64, 32), (128, 128), (32, 16)])
+def test_prepare_kernel_values_from_keys_and_queries_alone(dtype, d, rot):
     """The prepare kernel with values that are the keys as projected (the value pages get the unnormalised, unrotated keys)
-    and with rows of queries alone (a layer that reads another layer's cache): norm over the projection, rotation by halves."""
+    and with rows of queries alone (a layer that reads another layer's cache): norm over the projection, rotation by halves;
+    at a head size only the general form takes and at those of the form that gives a lane eight channels (bfloat16)."""
     from kestrel_amd.ops import core
 
     gen = torch.Generator().manual_seed(8)
-    n, H, G, d, rot, page = 21, 4, 2, 24, 12, 16
+    n, H, G, page = 21, 4, 2, 16
     eps = 1e-5
     places = list(range(3, 3 + n))
     freqs = plain.frequencies({"dims": rot, "base": 40.0})
@@ -347,7 +349,7 @@ def test_prepare_kernel_values_from_keys_and_queries_alone(dtype):
     q64, k64 = rows[:, :H * d].double(), rows[:, H * d:].double()
     want_q = plain.rotate_halves((plain.rms(q64, eps) * q_gain.double()).reshape(n, H, d), places, freqs).reshape(n, H * d)
     want_k = plain.rotate_halves((plain.rms(k64, eps) * k_gain.double()).reshape(n, G, d), places, freqs)
-    tol = dict(atol=2e-6, rtol=2e-6) if dtype == torch.float32 else dict(atol=2e-2, rtol=2e-2)
+    tol = dict(atol=5e-6, rtol=5e-6) if dtype == torch.float32 else dict(atol=2e-2, rtol=2e-2)
     _near(qk[:, :H * d], want_q, dtype, "queries", **tol)
     for t in range(n):
         slot = 5 + t
